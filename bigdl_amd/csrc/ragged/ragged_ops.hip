@@ -1,0 +1,307 @@
+// Row-wise kernels of the ragged engine: residual sum + grouped RMS norm, short causal convolution with per-sequence
+// state + per-head norm + rotary + paged append, clamped gated activation, HGRN2 gates / scan / output norm.
+// gfx950, wave64.  Everything that the engine keeps in 32 bits (residual, norms, angles, gates, recurrent state) is
+// float here whatever the activation type T is.
+#include "ragged_common.h"
+
+using namespace ragged;
+
+// ---------------------------------------------------------------------------------------------------------------
+// x <- w * groupnorm(alpha * x + y): the vector is cut into `groups` equal parts, each divided by its own root mean
+// square (eps inside the root).  One workgroup per (row, group).  x float in place; xa: the same values as T for the
+// matrix product that reads them next.  y may be null (a plain norm).  x_out may differ from x (the final norm).
+template <typename T>
+__global__ __launch_bounds__(256) void sum_group_norm_kernel(const float* __restrict__ x, const T* __restrict__ y,
+                                                             const float* __restrict__ w, float* __restrict__ x_out,
+                                                             T* __restrict__ xa, int D, int groups, float alpha, float eps) {
+  const int row = blockIdx.x / groups, g = blockIdx.x % groups, dg = D / groups;
+  const int64_t base = (int64_t)row * D + (int64_t)g * dg;
+  __shared__ float red[4];
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < dg; c += 256) {
+    float v = alpha * x[base + c] + (y ? to_f(y[base + c]) : 0.f);
+    ss += v * v;
+  }
+  ss = wave_sum(ss);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float r = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)dg + eps);
+  for (int c = threadIdx.x; c < dg; c += 256) {
+    float v = alpha * x[base + c] + (y ? to_f(y[base + c]) : 0.f);
+    v = v * r * w[g * dg + c];
+    if (x_out) x_out[base + c] = v;
+    if (xa) xa[base + c] = from_f<T>(v);
+  }
+}
+
+extern "C" int ragged_sum_group_norm(const float* x, const void* y, const float* w, float* x_out, void* xa, int64_t rows,
+                                     int D, int groups, float alpha, float eps, int dtype, hipStream_t st) {
+  if (rows <= 0 || D <= 0 || groups <= 0 || D % groups || rows * groups > 0x7fffffff) return -1;
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((sum_group_norm_kernel<T>), dim3((unsigned)(rows * groups)), dim3(256), 0, st, x,
+                                            (const T*)y, w, x_out, (T*)xa, D, groups, alpha, eps))
+  return RAGGED_LAUNCH_OK();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Short causal convolution over time per channel, then (optionally) RMS norm over groups of `gsize` channels with a
+// weight shared by all groups, then (optionally) rotation of the first `rot` channels of each group (pairs i, i + rot/2,
+// angle = position * inv_freq[i]), then a store into a dense float buffer or into cache pages.
+struct ConvHeadArgs {
+  const void* P;          // [T, ldp] projections of this step
+  int64_t ldp;
+  int col0;               // first column of this segment in P
+  const float* cw;        // [C, taps] taps of the whole convolved region, or null (no convolution)
+  int taps, C, ch0;       // ch0: this segment's first channel inside the convolved region
+  const void* state;      // [slots, taps - 1, C]: the last taps - 1 projected rows of every sequence
+  int ngroups, gsize;
+  const float* normw;     // [gsize] or null
+  float eps;
+  int rot;                // 0: no rotation
+  const float* inv_freq;  // [rot / 2]
+  float* out_dense;       // [T, ngroups * gsize] or null
+  void* pages;            // [num_pages, heads, PAGE, rowlen]
+  int rowlen, heads;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void conv_head_kernel(ConvHeadArgs a, Batch bt) {
+  extern __shared__ float smem[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t item = (int64_t)blockIdx.x * 4 + wave;
+  const bool live = item < (int64_t)bt.T * a.ngroups;
+  float* buf = smem + wave * a.gsize;
+  int t = 0, grp = 0, b = 0, pos = 0, past = 0, slot = 0;
+  if (live) {
+    t = (int)(item / a.ngroups);
+    grp = (int)(item % a.ngroups);
+    b = bt.tok_seq[t];
+    pos = bt.tok_pos[t];
+    past = bt.seq_past[b];
+    slot = bt.seq_slot[b];
+  }
+  const T* P = (const T*)a.P;
+  const T* S = (const T*)a.state;
+  float ss = 0.f;
+  if (live) {
+    for (int c = lane; c < a.gsize; c += 64) {
+      const int f = grp * a.gsize + c;           // channel inside the segment
+      float v;
+      if (a.cw) {
+        const int ch = a.ch0 + f;
+        v = 0.f;
+        for (int j = 0; j < a.taps; ++j) {
+          const int back = a.taps - 1 - j, pp = pos - back;
+          float u = 0.f;
+          if (pp >= past) u = to_f(P[(int64_t)(t - back) * a.ldp + a.col0 + f]);
+          else if (pp >= 0) u = to_f(S[((int64_t)slot * (a.taps - 1) + (pp - past + a.taps - 1)) * a.C + ch]);
+          v += a.cw[(int64_t)ch * a.taps + j] * u;
+        }
+      } else {
+        v = to_f(P[(int64_t)t * a.ldp + a.col0 + f]);
+      }
+      buf[c] = v;
+      ss += v * v;
+    }
+  }
+  if (a.normw) {
+    ss = wave_sum(ss);
+    const float r = 1.0f / sqrtf(ss / (float)a.gsize + a.eps);
+    if (live)
+      for (int c = lane; c < a.gsize; c += 64) buf[c] = buf[c] * r * a.normw[c];
+  }
+  __syncthreads();
+  if (!live) return;
+  const int half = a.rot >> 1;
+  for (int c = lane; c < a.gsize; c += 64) {
+    float v = buf[c];
+    if (c < a.rot) {
+      const int i = c < half ? c : c - half;
+      const float ang = (float)pos * a.inv_freq[i];
+      float sn, cs;
+      sincosf(ang, &sn, &cs);
+      v = c < half ? buf[c] * cs - buf[c + half] * sn : buf[c] * cs + buf[c - half] * sn;
+    }
+    const int f = grp * a.gsize + c;
+    if (a.out_dense) {
+      a.out_dense[(int64_t)t * a.ngroups * a.gsize + f] = v;
+    } else {
+      const int head = f / a.rowlen, off = f % a.rowlen;
+      const int page = bt.pages[(int64_t)b * bt.max_pages + pos / PAGE];
+      ((T*)a.pages)[(((int64_t)page * a.heads + head) * PAGE + (pos % PAGE)) * a.rowlen + off] = from_f<T>(v);
+    }
+  }
+}
+
+extern "C" int ragged_conv_head(ConvHeadArgs a, Batch bt, int dtype, hipStream_t st) {
+  if (bt.T <= 0 || a.ngroups <= 0 || a.gsize <= 0 || a.gsize > 2048) return -1;
+  if (a.cw && (a.taps < 1 || a.taps > 16 || (a.taps > 1 && !a.state))) return -1;
+  if (a.rot < 0 || (a.rot & 1) || a.rot > a.gsize || (a.rot && !a.inv_freq)) return -1;
+  if (!a.out_dense && (!a.pages || a.rowlen <= 0 || (a.ngroups * a.gsize) % a.rowlen || a.heads * a.rowlen != a.ngroups * a.gsize))
+    return -1;
+  const int64_t items = (int64_t)bt.T * a.ngroups;
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((conv_head_kernel<T>), dim3((unsigned)((items + 3) / 4)), dim3(256),
+                                            4 * a.gsize * sizeof(float), st, a, bt))
+  return RAGGED_LAUNCH_OK();
+}
+
+// The convolution's state after a step: projected rows of positions past + n - (taps - 1) .. past + n - 1 (zeros before
+// the sequence's start).  One thread per (sequence, channel) reads all it needs before it writes.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_state_kernel(const T* __restrict__ P, int64_t ldp, int col0, T* __restrict__ state,
+                                                         int taps, int C, Batch bt) {
+  const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (id >= (int64_t)bt.B * C) return;
+  const int b = (int)(id / C), ch = (int)(id % C);
+  const int start = bt.seq_start[b], n = bt.seq_start[b + 1] - start, past = bt.seq_past[b], slot = bt.seq_slot[b];
+  const int keep = taps - 1;
+  T vals[15];
+  for (int k = 0; k < keep; ++k) {
+    const int pp = past + n - keep + k;
+    T v = from_f<T>(0.f);
+    if (pp >= past) v = P[(int64_t)(start + pp - past) * ldp + col0 + ch];
+    else if (pp >= 0) v = state[((int64_t)slot * keep + (pp - past + keep)) * C + ch];
+    vals[k] = v;
+  }
+  for (int k = 0; k < keep; ++k) state[((int64_t)slot * keep + k) * C + ch] = vals[k];
+}
+
+extern "C" int ragged_conv_state(const void* P, int64_t ldp, int col0, void* state, int taps, int C, Batch bt, int dtype,
+                                 hipStream_t st) {
+  if (bt.B <= 0 || C <= 0 || taps < 2 || taps > 16) return -1;
+  const int64_t n = (int64_t)bt.B * C;
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((conv_state_kernel<T>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                                            (const T*)P, ldp, col0, (T*)state, taps, C, bt))
+  return RAGGED_LAUNCH_OK();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Clamped gated unit: g = min(gate, limit), u = clamp(up, -limit, limit), y = g * sigmoid(slope * g) * (u + 1).
+// GU holds [gate | up] per row.
+template <typename T>
+__global__ __launch_bounds__(256) void clamped_glu_kernel(const T* __restrict__ GU, T* __restrict__ out, int64_t rows, int F,
+                                                          float limit, float slope) {
+  const int64_t n = rows * F;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / F, c = i % F;
+    float g = fminf(to_f(GU[r * 2 * F + c]), limit);
+    float u = fminf(fmaxf(to_f(GU[r * 2 * F + F + c]), -limit), limit);
+    out[i] = from_f<T>(g * sigmoidf_(slope * g) * (u + 1.0f));
+  }
+}
+
+extern "C" int ragged_clamped_glu(const void* GU, void* out, int64_t rows, int F, float limit, float slope, int dtype,
+                                  hipStream_t st) {
+  if (rows <= 0 || F <= 0) return -1;
+  const int64_t n = rows * F;
+  const unsigned grid = (unsigned)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((clamped_glu_kernel<T>), dim3(grid), dim3(256), 0, st, (const T*)GU, (T*)out, rows, F,
+                                            limit, slope))
+  return RAGGED_LAUNCH_OK();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// HGRN2.  Gates: q = silu(q_proj), f = lower + (1 - lower) * sigmoid(f_proj + bias), both float [T, HD].
+template <typename T>
+__global__ __launch_bounds__(256) void hgrn2_gates_kernel(const T* __restrict__ P, int64_t ldp, int q0, int f0,
+                                                          const float* __restrict__ fb, const float* __restrict__ lower,
+                                                          float* __restrict__ qf, float* __restrict__ ff, int64_t rows, int HD) {
+  const int64_t n = rows * HD;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / HD;
+    const int c = (int)(i % HD);
+    const float q = to_f(P[r * ldp + q0 + c]);
+    qf[i] = q * sigmoidf_(q);
+    const float l = lower[c];
+    ff[i] = l + (1.0f - l) * sigmoidf_(to_f(P[r * ldp + f0 + c]) + fb[c]);
+  }
+}
+
+extern "C" int ragged_hgrn2_gates(const void* P, int64_t ldp, int q0, int f0, const float* fb, const float* lower, float* qf,
+                                  float* ff, int64_t rows, int HD, int dtype, hipStream_t st) {
+  if (rows <= 0 || HD <= 0) return -1;
+  const int64_t n = rows * HD;
+  const unsigned grid = (unsigned)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((hgrn2_gates_kernel<T>), dim3(grid), dim3(256), 0, st, (const T*)P, ldp, q0, f0, fb,
+                                            lower, qf, ff, rows, HD))
+  return RAGGED_LAUNCH_OK();
+}
+
+// Scan: per head S <- diag(f_t) S + (1 - f_t) v_t^T, o_t = S^T q_t, S float [d, vd] per (slot, head).
+// A wavefront owns 64 / R columns of S; R neighbouring lanes share a column and hold DR = ceil(d / R) <= 32 of its rows
+// in registers.  The wavefront walks the tokens of its sequence in order with no barrier: the only cross-lane step is
+// the sum of R partial dot products.  Grid: (column blocks, heads, sequences).
+constexpr int HG_DR = 32;
+
+template <typename T>
+__global__ __launch_bounds__(64) void hgrn2_scan_kernel(const float* __restrict__ qf, const float* __restrict__ ff,
+                                                        const T* __restrict__ P, int64_t ldp, int v0, float* __restrict__ state,
+                                                        float* __restrict__ out, int H, int d, int vd, int R, int DR, Batch bt) {
+  const int b = blockIdx.z, h = blockIdx.y, lane = threadIdx.x;
+  const int r = lane % R, col = blockIdx.x * (64 / R) + lane / R;
+  const int start = bt.seq_start[b], n = bt.seq_start[b + 1] - start, past = bt.seq_past[b], slot = bt.seq_slot[b];
+  const bool colok = col < vd;
+  const int row0 = r * DR;
+  float S[HG_DR];
+  float* sp = state + (((int64_t)slot * H + h) * d) * vd;
+#pragma unroll
+  for (int k = 0; k < HG_DR; ++k) {
+    const int row = row0 + k;
+    S[k] = (past > 0 && colok && k < DR && row < d) ? sp[(int64_t)row * vd + col] : 0.f;
+  }
+  const int HD = H * d;
+  for (int i = 0; i < n; ++i) {
+    const int64_t t = start + i;
+    const float* qrow = qf + t * HD + h * d;
+    const float* frow = ff + t * HD + h * d;
+    const float v = colok ? to_f(P[t * ldp + v0 + h * vd + col]) : 0.f;
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < HG_DR; ++k) {
+      const int row = row0 + k;
+      if (k < DR && row < d) {
+        const float f = frow[row];
+        S[k] = f * S[k] + (1.0f - f) * v;
+        acc += S[k] * qrow[row];
+      }
+    }
+    for (int o = 1; o < R; o <<= 1) acc += __shfl_xor(acc, o, 64);
+    if (r == 0 && colok) out[t * (int64_t)(H * vd) + h * vd + col] = acc;
+  }
+#pragma unroll
+  for (int k = 0; k < HG_DR; ++k) {
+    const int row = row0 + k;
+    if (colok && k < DR && row < d) sp[(int64_t)row * vd + col] = S[k];
+  }
+}
+
+extern "C" int ragged_hgrn2_scan(const float* qf, const float* ff, const void* P, int64_t ldp, int v0, float* state, float* out,
+                                 int H, int d, int vd, Batch bt, int dtype, hipStream_t st) {
+  if (bt.B <= 0 || H <= 0 || d <= 0 || vd <= 0 || d > HG_DR * 64) return -1;
+  int R = 1;
+  while (R * HG_DR < d) R <<= 1;
+  const int DR = (d + R - 1) / R, cols = 64 / R;
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((hgrn2_scan_kernel<T>), dim3((vd + cols - 1) / cols, H, bt.B), dim3(64), 0, st, qf, ff,
+                                            (const T*)P, ldp, v0, state, out, H, d, vd, R, DR, bt))
+  return RAGGED_LAUNCH_OK();
+}
+
+// RMS norm over rows of `n` floats with a weight (or none), output of type T.  One wavefront per row.
+template <typename T>
+__global__ __launch_bounds__(256) void row_norm_kernel(const float* __restrict__ x, const float* __restrict__ w, T* __restrict__ out,
+                                                       int64_t rows, int n, float eps) {
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  float ss = 0.f;
+  for (int c = lane; c < n; c += 64) { const float v = x[row * n + c]; ss += v * v; }
+  ss = wave_sum(ss);
+  const float r = 1.0f / sqrtf(ss / (float)n + eps);
+  for (int c = lane; c < n; c += 64) out[row * n + c] = from_f<T>(x[row * n + c] * r * (w ? w[c] : 1.0f));
+}
+
+extern "C" int ragged_row_norm(const float* x, const float* w, void* out, int64_t rows, int n, float eps, int dtype, hipStream_t st) {
+  if (rows <= 0 || n <= 0) return -1;
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((row_norm_kernel<T>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, x, w, (T*)out,
+                                            rows, n, eps))
+  return RAGGED_LAUNCH_OK();
+}

@@ -1228,3 +1228,25 @@ def is_native_arch(config_dict: dict, opt_in: Optional[bool] = None) -> bool:
         return True
     from transformers.models.auto.configuration_auto import CONFIG_MAPPING_NAMES
     return mt not in CONFIG_MAPPING_NAMES
+
+
+# ---------------------------------------------------------------------------------------------
+# designs that run on the ragged engine (models/ragged_engine.py): chosen by config.json's "architecture"
+# ---------------------------------------------------------------------------------------------
+def ragged_arch(config_dict: dict):
+    """The module that builds a ragged engine for this config (``read_config``, ``build_engine``, ``load``), or None."""
+    from . import lipizen
+    for mod in (lipizen,):
+        if config_dict.get("architecture") == mod.ARCHITECTURE:
+            return mod
+    return None
+
+
+def load_ragged_engine(path: str, dtype=torch.bfloat16, device="cuda"):
+    with open(os.path.join(path, "config.json")) as f:
+        cfg = json.load(f)
+    mod = ragged_arch(cfg)
+    if mod is None:
+        raise ValueError(f"{path}: config.json names no design of the ragged engine "
+                         f"(architecture = {cfg.get('architecture')!r})")
+    return mod.load(path, dtype, device)

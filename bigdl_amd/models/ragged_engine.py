@@ -1,0 +1,258 @@
+"""Ragged engine: decoder stacks whose layers are not all alike, stepped over a flat batch of token rows.
+
+``NativeDecoder`` runs families whose layers share one shape on a slot cache in fp16.  Designs that interleave kinds of
+token mixers (windowed attention with kept first tokens, score maps that are subtracted, layers that read another
+layer's keys and values, gated linear recurrences), that keep the residual stream in 32 bits, or that want prompts cut
+into arbitrary portions next to single decoded tokens run here instead:
+
+* a step takes ``[(slot, token ids), ...]``: any mix of prompt portions and single tokens, one row per token.  Every
+  product runs once over all rows; the mixers read ``BatchMeta`` (row -> sequence, position, pages);
+* keys / values live in 64-token pages of a ``PagedStatePool``, per-sequence state in its slots;
+* the mixers are described by small dataclasses whose fields are the design's constants, so a new design is a new list
+  of them (``models/lipizen.py`` builds one from a ``config.json``);
+* matrix products are the library's (bf16 inputs with 32-bit accumulation, or plain float32), everything between them
+  is ``ops/ragged.py``.
+"""
+from __future__ import annotations
+
+import math
+import time
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence
+
+import torch
+import torch.nn.functional as F
+
+from ..ops import ragged as R
+from .paged import PagedStatePool
+
+
+@dataclass
+class WindowAttention:
+    """Softmax attention over cache pages.  ``maps`` = 2: two score maps per head (queries / keys are [map 1 | map 2])
+    over the same values, combined as a1 - lam * a2 (differential attention)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    maps: int = 1
+    lam: float = 0.0               # weight of the second map
+    out_scale: float = 1.0         # after the per-head output norm
+    out_norm: bool = False         # each head's output divided by its root mean square (no weight)
+    conv_taps: int = 0             # short causal convolution behind the q / k / v projections (0: none)
+    qk_norm: bool = False          # RMS norm over ``dim`` with a weight shared by heads and maps, before rotation
+    rot_dims: int = 0              # leading channels of every map that are rotated (pairs i, i + rot_dims / 2)
+    rot_base: float = 10000.0
+    rot_factor: float = 1.0        # linear scaling: frequencies divided by this
+    window: int = 0                # 0: full causal attention
+    keep_first: int = 0            # the first tokens stay visible behind the window
+    gate: bool = False             # one sigmoid gate per head, from the mixer's input
+    kv_from: Optional[int] = None  # read this layer's cache instead of projecting keys / values
+
+
+@dataclass
+class Hgrn2:
+    """Gated linear recurrence with a matrix state per head: S <- diag(f) S + (1 - f) v^T, o = S^T q."""
+    heads: int
+    dim: int
+    vdim: int
+
+
+@dataclass
+class ClampedGlu:
+    """g = min(gate, limit), u = clamp(up, -limit, limit), y = g * sigmoid(slope * g) * (u + 1)"""
+    ff: int
+    limit: float
+    slope: float = 1.702
+
+
+@dataclass
+class RaggedConfig:
+    vocab: int
+    width: int
+    mixers: list                   # one mixer dataclass per layer
+    mlps: list                     # ClampedGlu or None per layer
+    norm_eps: float = 1e-6
+    norm_groups: int = 1
+    residual_alpha: float = 1.0    # x <- norm(alpha * x + sublayer(x))
+    logit_softcap: float = 0.0
+    name: str = "ragged"
+
+
+@dataclass
+class LayerTensors:
+    w_in: torch.Tensor                       # stacked input projections [rows, width], activation type
+    w_out: torch.Tensor
+    norm1: torch.Tensor
+    norm2: Optional[torch.Tensor] = None
+    conv_w: Optional[torch.Tensor] = None    # float [convolved channels, taps]
+    q_norm: Optional[torch.Tensor] = None
+    k_norm: Optional[torch.Tensor] = None
+    inv_freq: Optional[torch.Tensor] = None
+    f_bias: Optional[torch.Tensor] = None
+    lower: Optional[torch.Tensor] = None
+    o_norm: Optional[torch.Tensor] = None
+    w_gu: Optional[torch.Tensor] = None      # [gate; up]
+    w_down: Optional[torch.Tensor] = None
+
+
+def rotary_inv_freq(dims: int, base: float, factor: float) -> torch.Tensor:
+    """f_i = base^(-2 i / dims) / factor, i < dims / 2, evaluated in float32"""
+    i = torch.arange(dims // 2, dtype=torch.float32)
+    return (float(base) ** (-2.0 * i / dims)) / float(factor)
+
+
+class RaggedDecoder:
+    ragged = True                  # serving/continuous.py steps such an engine with mixed batches
+
+    def __init__(self, cfg: RaggedConfig, embed: torch.Tensor, layers: List[LayerTensors], final_norm: torch.Tensor,
+                 head: torch.Tensor, act_dtype=torch.bfloat16, device="cuda"):
+        self.cfg, self.embed, self.layers, self.final_norm, self.head = cfg, embed, layers, final_norm, head
+        self.act = act_dtype
+        self.device = torch.device(device)
+        self.ops = R.ops_for(self.device)
+        self.pool: Optional[PagedStatePool] = None
+        for li, m in enumerate(cfg.mixers):
+            if isinstance(m, WindowAttention) and m.kv_from is not None:
+                o = cfg.mixers[m.kv_from] if 0 <= m.kv_from < li else None
+                if not isinstance(o, WindowAttention) or o.kv_from is not None or \
+                        (o.kv_heads, o.dim, o.vdim, o.maps) != (m.kv_heads, m.dim, m.vdim, m.maps):
+                    raise ValueError(f"layer {li}: kv_from must name an earlier attention layer with keys of its own and "
+                                     "the same head layout")
+        self.first_cost = self.rest_cost_mean = self.peak_memory = 0.0
+
+    # ------------------------------------------------------------------ state
+    def state_specs(self):
+        specs = {}
+        for li, m in enumerate(self.cfg.mixers):
+            s = []
+            if isinstance(m, WindowAttention):
+                if m.kv_from is None:
+                    s.append(("kv", m.kv_heads, m.maps * m.dim, m.vdim))
+                if m.conv_taps > 1:
+                    s.append(("tail", m.conv_taps - 1, self._conv_channels(m)))
+            elif isinstance(m, Hgrn2):
+                s.append(("matrix", m.heads, m.dim, m.vdim))
+            specs[li] = s
+        return specs
+
+    @staticmethod
+    def _conv_channels(m: WindowAttention) -> int:
+        c = m.heads * m.maps * m.dim
+        if m.kv_from is None:
+            c += m.kv_heads * (m.maps * m.dim + m.vdim)
+        return c
+
+    def ensure_pool(self, max_tokens: int, slots: int) -> PagedStatePool:
+        p = self.pool
+        if p is None or p.num_pages * R.PAGE < max_tokens or p.slots < slots or p.len_of:
+            self.pool = PagedStatePool(self.state_specs(), max_tokens, slots, self.act, self.device)
+        return self.pool
+
+    # ------------------------------------------------------------------ layers
+    def _attention(self, li, m: WindowAttention, lt: LayerTensors, P, meta):
+        ops, pool, eps = self.ops, self.pool, self.cfg.norm_eps
+        cq = m.heads * m.maps * m.dim
+        ck = m.kv_heads * m.maps * m.dim
+        conv = dict(cw=lt.conv_w, taps=m.conv_taps, C=self._conv_channels(m), state=pool.tail.get(li)) if m.conv_taps else \
+            dict(cw=None, taps=0, C=0, state=None)
+        q = torch.empty(meta.T, cq, dtype=torch.float32, device=self.device)
+        ops.conv_head(P, 0, meta, ch0=0, ngroups=m.heads * m.maps, gsize=m.dim, normw=lt.q_norm, eps=eps, rot=m.rot_dims,
+                      inv_freq=lt.inv_freq, out_dense=q, **conv)
+        col = cq
+        if m.kv_from is None:
+            ops.conv_head(P, cq, meta, ch0=cq, ngroups=m.kv_heads * m.maps, gsize=m.dim, normw=lt.k_norm, eps=eps,
+                          rot=m.rot_dims, inv_freq=lt.inv_freq, pages=pool.k[li], **conv)
+            ops.conv_head(P, cq + ck, meta, ch0=cq + ck, ngroups=m.kv_heads, gsize=m.vdim, normw=None, eps=eps, rot=0,
+                          inv_freq=None, pages=pool.v[li], **conv)
+            col = cq + ck + m.kv_heads * m.vdim
+        if m.conv_taps > 1:
+            ops.conv_state(P, 0, pool.tail[li], m.conv_taps, conv["C"], meta)
+        src = li if m.kv_from is None else m.kv_from
+        return ops.paged_attn(q, pool.k[src], pool.v[src], meta, maps=m.maps, H=m.heads, G=m.kv_heads, d=m.dim, vd=m.vdim,
+                              window=m.window, keep_first=m.keep_first, scale=m.scale, lam=m.lam, out_scale=m.out_scale,
+                              out_norm=m.out_norm, eps=eps, gate=P if m.gate else None, gate0=col)
+
+    def _hgrn2(self, li, m: Hgrn2, lt: LayerTensors, P, meta):
+        ops = self.ops
+        hd = m.heads * m.dim
+        qf, ff = ops.hgrn2_gates(P, 0, hd, lt.f_bias, lt.lower, hd)
+        o = ops.hgrn2_scan(qf, ff, P, 2 * hd, self.pool.matrix[li], m.heads, m.dim, m.vdim, meta)
+        return ops.row_norm(o.view(meta.T * m.heads, m.vdim), lt.o_norm, self.cfg.norm_eps, self.act).view(meta.T, -1)
+
+    # ------------------------------------------------------------------ one step
+    @torch.no_grad()
+    def step(self, entries: Sequence[tuple], want: Optional[Sequence[Sequence[int]]] = None, collect: Optional[list] = None):
+        """``entries``: [(slot, token ids)] with slots from ``pool.admit()``; every entry continues its sequence by
+        these tokens.  ``want[i]``: indices into entry i's tokens whose logits are returned (default: the last one).
+        Returns float32 logits [wanted rows, vocab] in the order of entries and indices."""
+        cfg, ops, pool = self.cfg, self.ops, self.pool
+        seqs, ids = [], []
+        for slot, toks in entries:
+            if len(toks) == 0:
+                raise ValueError("an entry without tokens")
+            seqs.append((slot, pool.len_of[slot], len(toks), list(pool.reserve(slot, len(toks)))))
+            ids += list(toks)
+        meta = R.BatchMeta(seqs, self.device)
+        idt = torch.tensor(ids, dtype=torch.int64)
+        if self.device.type == "cuda":
+            idt = idt.pin_memory().to(self.device, non_blocking=True)
+        x = F.embedding(idt, self.embed).float()
+        xa = x.to(self.act)
+        for li, (m, mlp, lt) in enumerate(zip(cfg.mixers, cfg.mlps, self.layers)):
+            P = F.linear(xa, lt.w_in)
+            a = self._attention(li, m, lt, P, meta) if isinstance(m, WindowAttention) else self._hgrn2(li, m, lt, P, meta)
+            xa = ops.sum_group_norm(x, F.linear(a, lt.w_out), lt.norm1, cfg.norm_groups, cfg.residual_alpha, cfg.norm_eps, self.act)
+            if mlp is not None:
+                a = ops.clamped_glu(F.linear(xa, lt.w_gu), mlp.limit, mlp.slope)
+                xa = ops.sum_group_norm(x, F.linear(a, lt.w_down), lt.norm2, cfg.norm_groups, cfg.residual_alpha, cfg.norm_eps,
+                                        self.act)
+            if collect is not None:
+                collect.append(x.clone())
+        for slot, _, n, _ in seqs:
+            pool.commit(slot, n)
+        rows = []
+        for b, (_, _, n, _) in enumerate(seqs):
+            idx = [n - 1] if want is None else want[b]
+            if any(not 0 <= i < n for i in idx):
+                raise ValueError("a wanted index outside its entry")
+            rows += [meta.start[b] + i for i in idx]
+        if not rows:
+            return torch.empty(0, cfg.vocab, dtype=torch.float32, device=self.device)
+        xr = x[torch.tensor(rows, dtype=torch.int64, device=self.device)].contiguous()
+        xa = ops.sum_group_norm(xr, None, self.final_norm, cfg.norm_groups, 1.0, cfg.norm_eps, self.act)
+        logits = F.linear(xa, self.head).float()
+        if cfg.logit_softcap > 0:
+            logits = torch.tanh(logits / cfg.logit_softcap) * cfg.logit_softcap
+        return logits
+
+    # ------------------------------------------------------------------ generation
+    @torch.no_grad()
+    def generate(self, input_ids, max_new_tokens: int = 32, do_sample=False, temperature=1.0, top_k=0, top_p=1.0,
+                 eos_token_id=None, streamer=None, max_prefill_tokens: int = 4096, **_):
+        """Greedy / sampling generation for a [B, S] batch of equally long prompts (rows are independent sequences),
+        through the same scheduler that serves requests."""
+        from ..serving.continuous import generate_batch
+        ids = torch.as_tensor(input_ids)
+        prompts = [row.tolist() for row in ids.view(-1, ids.shape[-1])]
+        t0 = time.perf_counter()
+        outs = generate_batch(self, prompts, max_new_tokens=max_new_tokens, max_num_seqs=len(prompts),
+                              eos_token_id=eos_token_id, do_sample=do_sample, temperature=temperature, top_k=top_k, top_p=top_p)
+        dt = time.perf_counter() - t0
+        self.rest_cost_mean = dt / max(1, max_new_tokens)
+        width = max(len(o) for o in outs)
+        pad = eos_token_id if isinstance(eos_token_id, int) else 0
+        gen = torch.tensor([o + [pad] * (width - len(o)) for o in outs], dtype=torch.int64)
+        out = torch.cat([ids.view(-1, ids.shape[-1]).cpu(), gen], 1)
+        if streamer is not None:
+            streamer.put(ids.cpu())
+            streamer.put(gen)
+            streamer.end()
+        return out
+
+    def weight_bytes(self):
+        ts = [self.embed, self.head, self.final_norm]
+        for lt in self.layers:
+            ts += [t for t in vars(lt).values() if isinstance(t, torch.Tensor)]
+        return sum(t.numel() * t.element_size() for t in ts)

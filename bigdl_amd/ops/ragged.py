@@ -1,0 +1,419 @@
+"""Operations of the ragged engine (``bigdl_amd/models/ragged_engine.py``) over a flat batch of token rows.
+
+Two implementations of one interface:
+
+* ``HipOps``: the gfx950 kernels of ``libbigdl_ragged.so`` (``bigdl_amd/csrc/ragged``), loaded with ctypes and launched
+  on PyTorch's current stream.  The library is small and separate from ``libbigdl_hip.so`` so that a checkout without
+  built files compiles only what this engine needs (two translation units) the first time it is used.
+* ``TorchOps``: the same operations as unfused PyTorch statements, sequence by sequence.  It exists for host-side tests
+  of the engine's bookkeeping (pages, slots, portions) and is only ever chosen for tensors on the CPU; on a GPU the
+  kernels run or the call raises.
+
+Activations (``act``) are bfloat16 or float32; residual stream, norms, rotary angles, attention scores, gates and
+recurrent state are float32 in both.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+import os
+import subprocess
+import sys
+from pathlib import Path
+
+import torch
+import torch.nn.functional as F
+
+PAGE = 64
+_PKG = Path(__file__).resolve().parent.parent
+_SRC = _PKG / "csrc" / "ragged"
+_LIB_PATH = Path(os.environ.get("BIGDL_RAGGED_LIB") or _PKG / "lib" / "libbigdl_ragged.so")
+_LIB = None
+_DT = {torch.bfloat16: 1, torch.float32: 2}
+
+HIP_FLAGS = ["-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Wall", "-Wno-unused-function", "-DNDEBUG",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def build(force: bool = False) -> Path:
+    """Compile ``csrc/ragged/*.hip`` into ``lib/libbigdl_ragged.so`` (hipcc cross-compiles gfx950 without a GPU)."""
+    srcs = sorted(_SRC.glob("*.hip"))
+    deps = srcs + sorted(_SRC.glob("*.h"))
+    if not force and _LIB_PATH.exists() and all(p.stat().st_mtime <= _LIB_PATH.stat().st_mtime for p in deps):
+        return _LIB_PATH
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    _LIB_PATH.parent.mkdir(exist_ok=True)
+    tmp = _LIB_PATH.with_suffix(f".{os.getpid()}.tmp")
+    cmd = [hipcc, *HIP_FLAGS, "-shared", "-o", str(tmp), *map(str, srcs)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        sys.stderr.write(" ".join(cmd) + "\n" + r.stdout + r.stderr)
+        raise RuntimeError("building libbigdl_ragged.so failed")
+    os.replace(tmp, _LIB_PATH)
+    return _LIB_PATH
+
+
+class _Batch(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_void_p) for n in ("tok_seq", "tok_pos", "seq_start", "seq_past", "seq_slot", "pages")] + \
+               [(n, ctypes.c_int) for n in ("T", "B", "max_pages")]
+
+
+class _ConvHeadArgs(ctypes.Structure):
+    _fields_ = [("P", ctypes.c_void_p), ("ldp", ctypes.c_int64), ("col0", ctypes.c_int), ("cw", ctypes.c_void_p),
+                ("taps", ctypes.c_int), ("C", ctypes.c_int), ("ch0", ctypes.c_int), ("state", ctypes.c_void_p),
+                ("ngroups", ctypes.c_int), ("gsize", ctypes.c_int), ("normw", ctypes.c_void_p), ("eps", ctypes.c_float),
+                ("rot", ctypes.c_int), ("inv_freq", ctypes.c_void_p), ("out_dense", ctypes.c_void_p),
+                ("pages", ctypes.c_void_p), ("rowlen", ctypes.c_int), ("heads", ctypes.c_int)]
+
+
+class _AttnArgs(ctypes.Structure):
+    _fields_ = [("q", ctypes.c_void_p), ("kpages", ctypes.c_void_p), ("vpages", ctypes.c_void_p), ("out", ctypes.c_void_p),
+                ("gate", ctypes.c_void_p), ("ldg", ctypes.c_int64), ("gate0", ctypes.c_int), ("H", ctypes.c_int),
+                ("G", ctypes.c_int), ("d", ctypes.c_int), ("vd", ctypes.c_int), ("window", ctypes.c_int),
+                ("keep_first", ctypes.c_int), ("scale", ctypes.c_float), ("lam", ctypes.c_float),
+                ("out_scale", ctypes.c_float), ("out_norm", ctypes.c_int), ("eps", ctypes.c_float)]
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        if not _LIB_PATH.exists():
+            build()
+        L = ctypes.CDLL(str(_LIB_PATH))
+        vp, i64, ci, cf = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+        L.ragged_sum_group_norm.argtypes = [vp, vp, vp, vp, vp, i64, ci, ci, cf, cf, ci, vp]
+        L.ragged_conv_head.argtypes = [_ConvHeadArgs, _Batch, ci, vp]
+        L.ragged_conv_state.argtypes = [vp, i64, ci, vp, ci, ci, _Batch, ci, vp]
+        L.ragged_clamped_glu.argtypes = [vp, vp, i64, ci, cf, cf, ci, vp]
+        L.ragged_hgrn2_gates.argtypes = [vp, i64, ci, ci, vp, vp, vp, vp, i64, ci, ci, vp]
+        L.ragged_hgrn2_scan.argtypes = [vp, vp, vp, i64, ci, vp, vp, ci, ci, ci, _Batch, ci, vp]
+        L.ragged_row_norm.argtypes = [vp, vp, vp, i64, ci, cf, ci, vp]
+        L.ragged_paged_attn.argtypes = [_AttnArgs, _Batch, ci, ci, vp]
+        _LIB = L
+    return _LIB
+
+
+class BatchMeta:
+    """One step's batch: ``seqs`` is a list of (slot, past, n_new, page ids covering past + n_new tokens)."""
+
+    def __init__(self, seqs, device):
+        self.seqs = seqs
+        self.B = len(seqs)
+        self.start = [0]
+        for _, _, n, _ in seqs:
+            self.start.append(self.start[-1] + n)
+        self.T = self.start[-1]
+        self.max_pages = max(1, max(len(pg) for *_, pg in seqs))
+        tok_seq, tok_pos = [], []
+        for b, (_, past, n, _) in enumerate(seqs):
+            tok_seq += [b] * n
+            tok_pos += range(past, past + n)
+        flat = tok_seq + tok_pos + self.start + [s[1] for s in seqs] + [s[0] for s in seqs]
+        for *_, pg in seqs:
+            flat += list(pg) + [0] * (self.max_pages - len(pg))
+        buf = torch.tensor(flat, dtype=torch.int32)
+        if device.type == "cuda":
+            buf = buf.pin_memory().to(device, non_blocking=True)
+        self.buf = buf
+        T, B = self.T, self.B
+        o = [0, T, 2 * T, 2 * T + B + 1, 2 * T + 2 * B + 1, 2 * T + 3 * B + 1]
+        self.tok_seq, self.tok_pos = buf[o[0]:o[1]], buf[o[1]:o[2]]
+        self.seq_start, self.seq_past, self.seq_slot = buf[o[2]:o[3]], buf[o[3]:o[4]], buf[o[4]:o[5]]
+        self.pages = buf[o[5]:].view(B, self.max_pages)
+        self._c = None
+
+    def c(self):
+        if self._c is None:
+            self._c = _Batch(self.tok_seq.data_ptr(), self.tok_pos.data_ptr(), self.seq_start.data_ptr(),
+                             self.seq_past.data_ptr(), self.seq_slot.data_ptr(), self.pages.data_ptr(), self.T, self.B,
+                             self.max_pages)
+        return self._c
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ok(rc, what):
+    if rc != 0:
+        raise RuntimeError(f"{what}: the native launcher rejected the call (code {rc})")
+
+
+def _f32(*ts):
+    for t in ts:
+        if t is not None and (t.dtype != torch.float32 or not t.is_contiguous() or t.device.type != "cuda"):
+            raise ValueError("expected a contiguous float32 tensor on the HIP device")
+
+
+def _act(*ts):
+    for t in ts:
+        if t is not None and (t.dtype not in _DT or t.stride(-1) != 1 or t.device.type != "cuda"):
+            raise ValueError("expected a bfloat16 / float32 tensor with contiguous rows on the HIP device")
+
+
+def _page_check(meta: BatchMeta, pages: torch.Tensor):
+    need = max((p for *_, pg in meta.seqs for p in pg), default=0)
+    if need >= pages.shape[0] or pages.shape[2] != PAGE or not pages.is_contiguous():
+        raise ValueError("page ids outside the pool, or a pool that is not [pages, heads, 64, row]")
+    for _, past, n, pg in meta.seqs:
+        if len(pg) * PAGE < past + n:
+            raise ValueError("a sequence's pages do not cover its tokens")
+
+
+class HipOps:
+    """The kernels.  Every call checks shapes against what the kernel's indexing assumes before it launches."""
+    name = "hip"
+
+    def sum_group_norm(self, x, y, w, groups, alpha, eps, act, x_out=None, want_act=True):
+        _f32(x, w, x_out)
+        _act(y)
+        rows, D = x.shape
+        if y is not None and (y.shape != x.shape or not y.is_contiguous() or y.dtype != act):
+            raise ValueError("y must match x's shape and the activation type")
+        if w.numel() != D or D % groups:
+            raise ValueError("norm weight / group count do not fit the width")
+        xa = torch.empty(rows, D, dtype=act, device=x.device) if want_act else None
+        xo = x if x_out is None else x_out
+        _ok(lib().ragged_sum_group_norm(x.data_ptr(), None if y is None else y.data_ptr(), w.data_ptr(), xo.data_ptr(),
+                                        None if xa is None else xa.data_ptr(), rows, D, groups, alpha, eps, _DT[act],
+                                        _stream()), "sum_group_norm")
+        return xa
+
+    def conv_head(self, P, col0, meta, *, cw, taps, C, ch0, state, ngroups, gsize, normw, eps, rot, inv_freq,
+                  out_dense=None, pages=None):
+        _act(P, state, pages)
+        _f32(cw, normw, inv_freq, out_dense)
+        if P.dim() != 2 or P.shape[0] != meta.T or col0 < 0 or col0 + ngroups * gsize > P.shape[1]:
+            raise ValueError("segment outside the projection matrix")
+        a = _ConvHeadArgs()
+        a.P, a.ldp, a.col0 = P.data_ptr(), P.stride(0), col0
+        if cw is not None:
+            if cw.shape != (C, taps) or ch0 + ngroups * gsize > C:
+                raise ValueError("convolution taps do not cover the segment")
+            if taps > 1 and (state.dtype != P.dtype or state.shape[1:] != (taps - 1, C) or not state.is_contiguous()
+                             or max(s[0] for s in meta.seqs) >= state.shape[0]):
+                raise ValueError("convolution state does not fit")
+            a.cw, a.taps, a.C, a.ch0 = cw.data_ptr(), taps, C, ch0
+            a.state = None if state is None else state.data_ptr()
+        a.ngroups, a.gsize, a.eps = ngroups, gsize, eps
+        if normw is not None:
+            if normw.numel() != gsize:
+                raise ValueError("norm weight must have the group's size")
+            a.normw = normw.data_ptr()
+        if rot:
+            if inv_freq.numel() != rot // 2:
+                raise ValueError("one frequency per rotated pair")
+            a.rot, a.inv_freq = rot, inv_freq.data_ptr()
+        if out_dense is not None:
+            if out_dense.shape != (meta.T, ngroups * gsize):
+                raise ValueError("dense output shape")
+            a.out_dense = out_dense.data_ptr()
+        else:
+            _page_check(meta, pages)
+            heads, rowlen = pages.shape[1], pages.shape[3]
+            if pages.dtype != P.dtype or heads * rowlen != ngroups * gsize:
+                raise ValueError("cache pages do not fit the segment")
+            a.pages, a.rowlen, a.heads = pages.data_ptr(), rowlen, heads
+        _ok(lib().ragged_conv_head(a, meta.c(), _DT[P.dtype], _stream()), "conv_head")
+
+    def conv_state(self, P, col0, state, taps, C, meta):
+        _act(P, state)
+        if P.shape[0] != meta.T or col0 + C > P.shape[1] or state.shape[1:] != (taps - 1, C) or state.dtype != P.dtype \
+                or not state.is_contiguous() or max(s[0] for s in meta.seqs) >= state.shape[0]:
+            raise ValueError("convolution state does not fit")
+        _ok(lib().ragged_conv_state(P.data_ptr(), P.stride(0), col0, state.data_ptr(), taps, C, meta.c(), _DT[P.dtype],
+                                    _stream()), "conv_state")
+
+    def clamped_glu(self, GU, limit, slope):
+        _act(GU)
+        if not GU.is_contiguous() or GU.shape[1] % 2:
+            raise ValueError("[gate | up] rows expected")
+        rows, F2 = GU.shape
+        out = torch.empty(rows, F2 // 2, dtype=GU.dtype, device=GU.device)
+        _ok(lib().ragged_clamped_glu(GU.data_ptr(), out.data_ptr(), rows, F2 // 2, limit, slope, _DT[GU.dtype], _stream()),
+            "clamped_glu")
+        return out
+
+    def hgrn2_gates(self, P, q0, f0, fb, lower, HD):
+        _act(P)
+        _f32(fb, lower)
+        if max(q0, f0) + HD > P.shape[1] or fb.numel() != HD or lower.numel() != HD:
+            raise ValueError("gate segments outside the projection matrix")
+        rows = P.shape[0]
+        qf = torch.empty(rows, HD, dtype=torch.float32, device=P.device)
+        ff = torch.empty_like(qf)
+        _ok(lib().ragged_hgrn2_gates(P.data_ptr(), P.stride(0), q0, f0, fb.data_ptr(), lower.data_ptr(), qf.data_ptr(),
+                                     ff.data_ptr(), rows, HD, _DT[P.dtype], _stream()), "hgrn2_gates")
+        return qf, ff
+
+    def hgrn2_scan(self, qf, ff, P, v0, state, H, d, vd, meta):
+        _f32(qf, ff, state)
+        _act(P)
+        if qf.shape != (meta.T, H * d) or ff.shape != qf.shape or v0 + H * vd > P.shape[1] or P.shape[0] != meta.T \
+                or state.shape[1:] != (H, d, vd) or max(s[0] for s in meta.seqs) >= state.shape[0]:
+            raise ValueError("recurrent state / gates do not fit")
+        out = torch.empty(meta.T, H * vd, dtype=torch.float32, device=P.device)
+        _ok(lib().ragged_hgrn2_scan(qf.data_ptr(), ff.data_ptr(), P.data_ptr(), P.stride(0), v0, state.data_ptr(),
+                                    out.data_ptr(), H, d, vd, meta.c(), _DT[P.dtype], _stream()), "hgrn2_scan")
+        return out
+
+    def row_norm(self, x, w, eps, act):
+        _f32(x, w)
+        n = x.shape[-1]
+        if w is not None and w.numel() != n:
+            raise ValueError("norm weight size")
+        out = torch.empty(x.shape, dtype=act, device=x.device)
+        _ok(lib().ragged_row_norm(x.data_ptr(), None if w is None else w.data_ptr(), out.data_ptr(), x.numel() // n, n, eps,
+                                  _DT[act], _stream()), "row_norm")
+        return out
+
+    def paged_attn(self, q, kpages, vpages, meta, *, maps, H, G, d, vd, window, keep_first, scale, lam, out_scale, out_norm,
+                   eps, gate=None, gate0=0):
+        _f32(q)
+        _act(kpages, vpages, gate)
+        _page_check(meta, kpages)
+        _page_check(meta, vpages)
+        if q.shape != (meta.T, H * maps * d) or kpages.shape[1:] != (G, PAGE, maps * d) or vpages.shape[1:] != (G, PAGE, vd) \
+                or kpages.dtype != vpages.dtype or kpages.shape[0] != vpages.shape[0]:
+            raise ValueError("queries / cache pages do not fit the head layout")
+        out = torch.empty(meta.T, H * vd, dtype=kpages.dtype, device=q.device)
+        a = _AttnArgs()
+        a.q, a.kpages, a.vpages, a.out = q.data_ptr(), kpages.data_ptr(), vpages.data_ptr(), out.data_ptr()
+        if gate is not None:
+            if gate.shape[0] != meta.T or gate0 + H > gate.shape[1] or gate.dtype != kpages.dtype:
+                raise ValueError("gate columns outside the projection matrix")
+            a.gate, a.ldg, a.gate0 = gate.data_ptr(), gate.stride(0), gate0
+        a.H, a.G, a.d, a.vd, a.window, a.keep_first = H, G, d, vd, window, keep_first
+        a.scale, a.lam, a.out_scale, a.out_norm, a.eps = scale, lam, out_scale, int(out_norm), eps
+        _ok(lib().ragged_paged_attn(a, meta.c(), maps, _DT[kpages.dtype], _stream()), "paged_attn")
+        return out
+
+
+class TorchOps:
+    """The same interface as unfused PyTorch statements (host-side tests of the engine's bookkeeping)."""
+    name = "torch"
+
+    def sum_group_norm(self, x, y, w, groups, alpha, eps, act, x_out=None, want_act=True):
+        v = alpha * x if y is None else alpha * x + y.float()
+        g = v.view(v.shape[0], groups, -1)
+        g = g / torch.sqrt(g.pow(2).mean(-1, keepdim=True) + eps)
+        v = g.reshape(v.shape) * w
+        (x if x_out is None else x_out).copy_(v)
+        return v.to(act) if want_act else None
+
+    def _segment(self, P, col0, meta, cw, taps, C, ch0, state, width):
+        """convolved (or plain) float rows of a segment"""
+        u = P[:, col0:col0 + width].float()
+        if cw is None:
+            return u
+        out = torch.empty_like(u)
+        wseg = cw[ch0:ch0 + width]
+        for b, (slot, past, n, _) in enumerate(meta.seqs):
+            s0 = meta.start[b]
+            hist = state[slot, :, ch0:ch0 + width].float() if taps > 1 else u[:0]
+            if past < taps - 1:
+                hist = hist.clone()
+                hist[: taps - 1 - past] = 0
+            full = torch.cat([hist, u[s0:s0 + n]], 0)
+            acc = torch.zeros(n, width, dtype=torch.float32, device=P.device)
+            for j in range(taps):
+                acc += wseg[:, j] * full[j:j + n]
+            out[s0:s0 + n] = acc
+        return out
+
+    def conv_head(self, P, col0, meta, *, cw, taps, C, ch0, state, ngroups, gsize, normw, eps, rot, inv_freq,
+                  out_dense=None, pages=None):
+        width = ngroups * gsize
+        v = self._segment(P, col0, meta, cw, taps, C, ch0, state, width).view(meta.T, ngroups, gsize)
+        if normw is not None:
+            v = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps) * normw
+        if rot:
+            half = rot // 2
+            ang = meta.tok_pos.to(P.device).float()[:, None] * inv_freq[None]
+            c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
+            a, b2 = v[..., :half], v[..., half:rot]
+            v = torch.cat([a * c - b2 * s, b2 * c + a * s, v[..., rot:]], -1)
+        v = v.reshape(meta.T, width)
+        if out_dense is not None:
+            out_dense.copy_(v)
+            return
+        heads, rowlen = pages.shape[1], pages.shape[3]
+        v = v.view(meta.T, heads, rowlen).to(pages.dtype)
+        for b, (slot, past, n, pg) in enumerate(meta.seqs):
+            for i in range(n):
+                pos = past + i
+                pages[pg[pos // PAGE], :, pos % PAGE] = v[meta.start[b] + i]
+
+    def conv_state(self, P, col0, state, taps, C, meta):
+        keep = taps - 1
+        for b, (slot, past, n, _) in enumerate(meta.seqs):
+            old = state[slot].clone()
+            if past < keep:
+                old[: keep - past] = 0
+            full = torch.cat([old, P[meta.start[b]:meta.start[b] + n, col0:col0 + C]], 0)
+            state[slot] = full[-keep:]
+
+    def clamped_glu(self, GU, limit, slope):
+        f = GU.shape[1] // 2
+        g = GU[:, :f].float().clamp(max=limit)
+        u = GU[:, f:].float().clamp(-limit, limit)
+        return (g * torch.sigmoid(slope * g) * (u + 1)).to(GU.dtype)
+
+    def hgrn2_gates(self, P, q0, f0, fb, lower, HD):
+        q = P[:, q0:q0 + HD].float()
+        f = lower + (1 - lower) * torch.sigmoid(P[:, f0:f0 + HD].float() + fb)
+        return q * torch.sigmoid(q), f
+
+    def hgrn2_scan(self, qf, ff, P, v0, state, H, d, vd, meta):
+        out = torch.empty(meta.T, H * vd, dtype=torch.float32, device=P.device)
+        for b, (slot, past, n, _) in enumerate(meta.seqs):
+            S = state[slot].clone() if past > 0 else torch.zeros_like(state[slot])
+            for i in range(n):
+                t = meta.start[b] + i
+                f = ff[t].view(H, d, 1)
+                S = f * S + (1 - f) * P[t, v0:v0 + H * vd].float().view(H, 1, vd)
+                out[t] = (S * qf[t].view(H, d, 1)).sum(1).reshape(-1)
+            state[slot] = S
+        return out
+
+    def row_norm(self, x, w, eps, act):
+        v = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+        return (v if w is None else v * w).to(act)
+
+    def paged_attn(self, q, kpages, vpages, meta, *, maps, H, G, d, vd, window, keep_first, scale, lam, out_scale, out_norm,
+                   eps, gate=None, gate0=0):
+        out = torch.empty(meta.T, H * vd, dtype=torch.float32, device=q.device)
+        q = q.view(meta.T, H, maps, d)
+        for b, (slot, past, n, pg) in enumerate(meta.seqs):
+            L = past + n
+            idx = torch.tensor(pg, dtype=torch.long, device=q.device)
+            k = kpages[idx].float().permute(1, 0, 2, 3).reshape(G, -1, maps, d)[:, :L]       # [G, L, maps, d]
+            v = vpages[idx].float().permute(1, 0, 2, 3).reshape(G, -1, vd)[:, :L]
+            i = torch.arange(past, L, device=q.device)[:, None]
+            j = torch.arange(L, device=q.device)[None]
+            vis = j <= i
+            if window > 0:
+                vis &= (i - j < window) | (j < keep_first)
+            qs = q[meta.start[b]:meta.start[b] + n]
+            rep = H // G
+            o = None
+            for mp in range(maps):
+                s = torch.einsum("thd,hld->htl", qs[:, :, mp], k[:, :, mp].repeat_interleave(rep, 0)) * scale
+                a = torch.softmax(s.masked_fill(~vis, float("-inf")), -1) @ v.repeat_interleave(rep, 0)   # [H, n, vd]
+                o = a if mp == 0 else o - lam * a
+            o = o.permute(1, 0, 2)
+            if out_norm:
+                o = o / torch.sqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+            out[meta.start[b]:meta.start[b] + n] = (o * out_scale).reshape(n, H * vd)
+        if gate is not None:
+            out = (out.view(meta.T, H, vd) * torch.sigmoid(gate[:, gate0:gate0 + H].float())[:, :, None]).view(meta.T, H * vd)
+        return out.to(kpages.dtype)
+
+
+def ops_for(device) -> object:
+    """The kernels for a GPU, the PyTorch statements for the CPU.  A GPU never gets the latter."""
+    device = torch.device(device)
+    if device.type == "cuda":
+        lib()
+        return HipOps()
+    return TorchOps()
