@@ -10,6 +10,12 @@ import sys
 
 def _load(path, family, low_bit):
     import torch
+    if os.path.isdir(path) and not any(os.path.exists(os.path.join(path, f)) for f in
+                                       ("tokenizer.json", "tokenizer.model", "tokenizer_config.json", "vocab.json")):
+        # a checkpoint without a tokenizer: prompts are given as token ids (--prompt-ids), tokens come back as ids
+        from ..transformers import AutoModelForCausalLM
+        model = AutoModelForCausalLM.from_pretrained(path, load_in_low_bit=low_bit)
+        return model.to("cuda" if torch.cuda.is_available() else "cpu"), None
     if os.path.isdir(path):
         from ..transformers import AutoModelForCausalLM
         from transformers import AutoTokenizer
@@ -28,6 +34,14 @@ def _load(path, family, low_bit):
 
 def _complete(model, tok, prompt, n_predict, temperature, stream=True):
     import torch
+    if tok is None:
+        ids = torch.tensor([[int(t) for t in prompt.replace(",", " ").split()]])
+        kw = dict(do_sample=True, temperature=temperature) if temperature and temperature > 0 else dict(do_sample=False)
+        out = model.generate(ids, max_new_tokens=n_predict, **kw)
+        text = " ".join(str(int(t)) for t in out[0, ids.shape[1]:])
+        if stream:
+            print(text, end="")
+        return text
     from transformers import TextStreamer
     ids = tok(prompt, return_tensors="pt").input_ids.to(next(model.parameters()).device)
     streamer = TextStreamer(tok, skip_prompt=True, skip_special_tokens=True) if stream else None
@@ -50,8 +64,13 @@ def _parser(desc):
 
 def main(argv=None):
     ap = _parser("llm-cli: run a prompt through a low-bit model")
-    ap.add_argument("-p", "--prompt", required=True)
+    ap.add_argument("-p", "--prompt", help="text, or token ids when the checkpoint has no tokenizer")
+    ap.add_argument("--prompt-ids", help="token ids separated by spaces or commas (checkpoints without a tokenizer)")
     a = ap.parse_args(argv)
+    if a.prompt is None and a.prompt_ids is None:
+        ap.error("one of --prompt / --prompt-ids is required")
+    if a.prompt is None:
+        a.prompt = a.prompt_ids
     if a.threads:
         import torch
         torch.set_num_threads(a.threads)

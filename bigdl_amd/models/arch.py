@@ -1250,3 +1250,50 @@ def load_ragged_engine(path: str, dtype=torch.bfloat16, device="cuda"):
         raise ValueError(f"{path}: config.json names no design of the ragged engine "
                          f"(architecture = {cfg.get('architecture')!r})")
     return mod.load(path, dtype, device)
+
+
+class RaggedCausalLM:
+    """What ``AutoModelForCausalLM.from_pretrained`` returns for a design of the ragged engine: the checkpoint's tensors
+    on the host until ``.to(device)`` builds the engine (kernels on a GPU; on the CPU the unfused statements that the
+    host-side tests use).  ``generate`` goes through the continuous batcher, as serving does."""
+
+    def __init__(self, path: str, dtype=None):
+        with open(os.path.join(path, "config.json")) as f:
+            self.source_config = json.load(f)
+        self.mod = ragged_arch(self.source_config)
+        if self.mod is None:
+            raise ValueError(f"{path}: no design of the ragged engine")
+        self.config = self.mod.read_config(self.source_config)
+        self.sd = load_checkpoint_tensors(path)
+        self.dtype = dtype or torch.bfloat16
+        self.engine = None
+        self.device = torch.device("cpu")
+
+    def to(self, device=None, dtype=None):
+        if isinstance(device, torch.dtype):
+            device, dtype = None, device
+        if dtype is not None:
+            self.dtype = dtype
+        if device is not None:
+            self.device = torch.device(device)
+        self.engine = self.mod.build_engine(self.mod.read_config(self.source_config), self.sd, self.dtype, self.device)
+        return self
+
+    def half(self):
+        return self
+
+    def float(self):
+        self.dtype = torch.float32
+        return self.to(self.device) if self.engine is not None else self
+
+    def eval(self):
+        return self
+
+    def parameters(self):
+        yield torch.empty(0, device=self.device)
+
+    @torch.no_grad()
+    def generate(self, input_ids, max_new_tokens: int = 32, **kw):
+        if self.engine is None:
+            self.to(self.device)
+        return self.engine.generate(input_ids, max_new_tokens=max_new_tokens, **kw)

@@ -17,6 +17,12 @@ prompt's rows, so the step costs one read of the weights instead of two.  Prompt
 are admitted in chunks of that many tokens, one chunk per step (the reference's partial prefill,
 python/llm/src/ipex_llm/transformers/pipeline_parallel.py:621-700), so a long prompt delays the running sequences by
 one chunk's time per token instead of stalling them for the whole prompt.
+
+Engines that step a flat batch of token rows (``engine.ragged``, ``models/ragged_engine.py``) need none of the special
+passes: every iteration is ONE ``engine.step`` whose rows are the next token of every running request plus prompt
+portions of the requests being admitted, up to ``max_prefill_tokens`` rows.  Their cache is a page pool sized in tokens
+(``max_live_tokens``), so a request is admitted when a state slot is free and the pages for its prompt and its
+``max_new_tokens`` are not already promised to the live requests.
 """
 from __future__ import annotations
 
@@ -56,8 +62,9 @@ class ContinuousBatcher:
     def __init__(self, engine, max_num_seqs: int = 8, max_seq_len: int = 4096, kv_fp8: bool = False,
                  max_prefill_per_step: int = 8, on_token: Optional[Callable[[SeqRequest, int], None]] = None,
                  piggyback: Optional[bool] = None, dense_prefill_cache: Optional[bool] = None,
-                 max_prefill_tokens: Optional[int] = 4096):
+                 max_prefill_tokens: Optional[int] = 4096, max_live_tokens: Optional[int] = None):
         self.engine = engine
+        self.ragged = bool(getattr(engine, "ragged", False))
         self.max_num_seqs = max_num_seqs
         self.max_seq_len = max_seq_len
         self.max_prefill_per_step = max(1, max_prefill_per_step)
@@ -65,6 +72,19 @@ class ContinuousBatcher:
         self.waiting: collections.deque = collections.deque()
         self.running: Dict[int, SeqRequest] = {}
         self.free_slots = list(range(max_num_seqs))[::-1]
+        self.steps = 0
+        self.generated = 0
+        self.mixed_steps = 0
+        self.packed_prompts = 0
+        self.max_prefill_tokens = max_prefill_tokens
+        self._prefilling = None
+        if self.ragged:
+            # page pool + state slots instead of the slot cache; see _step_ragged
+            self.pool = engine.ensure_pool(max_live_tokens or max_num_seqs * max_seq_len, max_num_seqs)
+            self.cache = None
+            self._admitting: List[list] = []           # [request, tokens of its prompt already in the cache]
+            self._promised = 0                         # pages promised to live requests (prompt + max_new_tokens)
+            return
         cache = engine.ensure_cache(max_num_seqs, max_seq_len, fp8=kv_fp8)
         cache.enable_slots()
         self.cache = cache
@@ -97,22 +117,31 @@ class ContinuousBatcher:
     def submit(self, req: SeqRequest) -> SeqRequest:
         if len(req.input_ids) == 0:
             raise ValueError(f"request {req.request_id}: empty prompt")
-        if len(req.input_ids) + req.max_new_tokens > self.cache.capacity:
-            raise ValueError(f"request {req.request_id}: prompt + max_new_tokens exceeds the slot capacity "
-                             f"({self.cache.capacity})")
+        capacity = self.pool.num_pages * 64 if self.ragged else self.cache.capacity
+        if len(req.input_ids) + req.max_new_tokens > capacity:
+            raise ValueError(f"request {req.request_id}: prompt + max_new_tokens exceeds the "
+                             f"{'page pool' if self.ragged else 'slot capacity'} ({capacity})")
         if isinstance(req.eos_token_id, int):
             req.eos_token_id = [req.eos_token_id]
         self.waiting.append(req)
         return req
 
     def has_work(self) -> bool:
-        return bool(self.waiting or self.running or self._prefilling)
+        return bool(self.waiting or self.running or self._prefilling or (self.ragged and self._admitting))
 
     def fail_all(self, reason: str = "error"):
         """After an exception inside ``step``: finish every admitted request (running, being prefilled) with
         ``finish_reason = reason``, free their slots and leave the batcher ready for new work.  Returns the failed
         requests; waiting requests stay queued.  Without this a failing step leaves ``has_work()`` true for ever."""
         failed = list(self.running.values())
+        if self.ragged:
+            failed += [r for r, _ in self._admitting]
+            self._admitting = []
+            now = time.perf_counter()
+            for req in failed:
+                req.finished, req.finish_reason, req.finish_time = True, reason, now
+                self._release_ragged(req)
+            return failed
         if self._prefilling is not None:
             failed.append(self._prefilling[0])
             self._prefilling = None
@@ -154,6 +183,9 @@ class ContinuousBatcher:
             self.on_token(req, token)
         if req.finished:
             req.finish_time = now
+            if self.ragged:
+                self._release_ragged(req)
+                return
             self.cache.set_active(req.slot, False)
             self.running.pop(req.slot, None)
             self.free_slots.append(req.slot)
@@ -233,8 +265,69 @@ class ContinuousBatcher:
         self.packed_mixed_steps += 1
         return True
 
+    # ------------------------------------------------------------------ ragged engines
+    @staticmethod
+    def _pages_for(req: SeqRequest) -> int:
+        return (len(req.input_ids) + req.max_new_tokens + 63) // 64
+
+    def _release_ragged(self, req: SeqRequest):
+        if req.slot is not None and req.slot >= 0 and req.slot in self.pool.len_of:
+            self.pool.release(req.slot)
+            self._promised -= self._pages_for(req)
+        self.running.pop(req.slot, None)
+        req.slot = -1
+
+    def _step_ragged(self) -> Dict[str, int]:
+        """One ``engine.step`` over the next token of every running request and prompt portions of the requests being
+        admitted (oldest first, ``max_prefill_tokens`` prompt rows per step)."""
+        eng, pool, out = self.engine, self.pool, {}
+        while self.waiting and pool.free_slots and len(self._admitting) < self.max_prefill_per_step \
+                and self._promised + self._pages_for(self.waiting[0]) <= pool.num_pages:
+            req = self.waiting.popleft()
+            req.slot = pool.admit()
+            self._promised += self._pages_for(req)
+            self._admitting.append([req, 0])
+        entries, want, who = [], [], []
+        for slot, req in self.running.items():
+            entries.append((slot, [req.output_ids[-1]]))
+            want.append([0])
+            who.append(req)
+        budget = self.max_prefill_tokens or (1 << 30)
+        started = []
+        for item in self._admitting:
+            if budget <= 0:
+                break
+            req, done = item
+            n = min(len(req.input_ids) - done, budget)
+            budget -= n
+            entries.append((req.slot, req.input_ids[done:done + n]))
+            item[1] = done + n
+            if item[1] == len(req.input_ids):
+                want.append([n - 1])
+                who.append(req)
+                started.append(req)
+            else:
+                want.append([])
+        if not entries:
+            return out
+        if len(entries) > 1 and any(len(t) > 1 for _, t in entries):
+            self.mixed_steps += 1
+        logits = eng.step(entries, want)
+        greedy = logits.argmax(-1).tolist() if logits.shape[0] else []       # one device sync per iteration
+        now = time.perf_counter()
+        self._admitting = [it for it in self._admitting if it[1] < len(it[0].input_ids)]
+        for req in started:
+            self.running[req.slot] = req
+        for row, req in enumerate(who):
+            tok = self._pick(req, logits[row]) if req.do_sample else greedy[row]
+            self._emit(req, tok, now, out)
+        self.steps += 1
+        return out
+
     def step(self) -> Dict[str, int]:
         """Admit, decode once, return {request_id: new token}."""
+        if self.ragged:
+            return self._step_ragged()
         eng, out = self.engine, {}
         tokens = self._token_buffer()
         admitted = 0
@@ -290,6 +383,7 @@ def generate_batch(engine, prompts: List[List[int]], max_new_tokens: int = 32, m
     """Run ``prompts`` (token id lists of any lengths) through a ``ContinuousBatcher``; returns the new tokens of
     each prompt in order."""
     cap = max(len(p) for p in prompts) + max_new_tokens + 1
+    cap = (cap + 63) // 64 * 64
     cb = ContinuousBatcher(engine, max_num_seqs=min(max_num_seqs, len(prompts)), max_seq_len=cap, kv_fp8=kv_fp8,
                            max_prefill_per_step=max_num_seqs)
     reqs = [cb.submit(SeqRequest(str(i), list(p), max_new_tokens=max_new_tokens, eos_token_id=eos_token_id, **sampling))

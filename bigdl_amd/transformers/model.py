@@ -212,7 +212,10 @@ class _BaseAutoModelClass:
         native_engine = kwargs.pop("native_engine", None)
         if not bigdl_transformers_low_bit and isinstance(pretrained_model_name_or_path, str) \
                 and os.path.isdir(pretrained_model_name_or_path):
-            from ..models.arch import NativeCausalLM, is_native_arch
+            from ..models.arch import NativeCausalLM, RaggedCausalLM, is_native_arch, ragged_arch
+            if ragged_arch(config_dict) is not None:
+                # designs of the ragged engine (mixed layer kinds, paged cache): chosen by config.json's "architecture"
+                return RaggedCausalLM(pretrained_model_name_or_path, kwargs.get("torch_dtype", kwargs.get("dtype")))
             if is_native_arch(config_dict, native_engine):
                 # families HuggingFace only has as remote code (chatglm, baichuan, qwen v1, internlm, minicpm, ...):
                 # loaded through their weight-name map into the native engine, no remote code is executed
