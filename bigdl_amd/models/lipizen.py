@@ -107,3 +107,71 @@ def load(path: str, dtype=torch.bfloat16, device="cuda") -> RaggedDecoder:
     if not is_lipizen(config):
         raise ValueError(f"{path}: not a {ARCHITECTURE} checkpoint")
     return build_engine(read_config(config), load_checkpoint_tensors(path), dtype, device)
+
+
+def example_config(width=2048, layers=16, heads=16, kv_heads=4, dim=64, vdim=128, ff=5632, vocab=32000, window=1024,
+                   keep_first=4, conv=4, rec_heads=16, rec_dim=128, groups=4) -> dict:
+    """A config.json of this design at the proportions of a real model: of every four layers two attention layers with
+    keys of their own, one HGRN2 layer without a feed-forward, one attention layer that reads the cache of the layer
+    before the recurrence.  For benchmarks and smoke tests (random weights)."""
+    def attn(kv_from=None):
+        m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "diff": 0.5, "scale": dim ** -0.5, "conv": conv,
+             "mask": {"size": window, "keep_first": keep_first},
+             "rot": {"dims": dim // 2, "base": 10000.0, "scaling": {"factor": 2.0}}}
+        if kv_from is not None:
+            m["kv_from"] = kv_from
+        return {"type": "attention", "mixer": m, "mlp": {"kind": "dense", "ff": ff, "limit": 7.0}}
+    out = []
+    for i in range(layers):
+        if i % 4 == 2:
+            out.append({"type": "hgrn2", "mixer": {"heads": rec_heads, "dim": rec_dim, "vdim": rec_dim}, "mlp": None})
+        elif i % 4 == 3:
+            out.append(attn(kv_from=i - 2))
+        else:
+            out.append(attn())
+    return {"architecture": ARCHITECTURE, "layers": out, "logit_softcap": 30.0, "norm": {"eps": 1e-6, "groups": groups},
+            "postln_alpha": 2.0, "vocab": vocab, "width": width}
+
+
+def random_state_dict(config: dict, device="cuda", seed: int = 0) -> dict:
+    """Random checkpoint tensors (bfloat16, created on ``device``) with the names and shapes the design gives them."""
+    dev = torch.device(device)
+    g = torch.Generator(device=dev).manual_seed(seed)
+    D = config["width"]
+
+    def mat(n, k, s=1.0):
+        return (torch.randn(n, k, device=dev, generator=g) * (s / math.sqrt(k))).to(torch.bfloat16)
+
+    def vec(n, mean=0.0, s=0.1):
+        return (mean + s * torch.randn(n, device=dev, generator=g)).to(torch.bfloat16)
+
+    sd = {"embed": mat(config["vocab"], D, math.sqrt(D)), "final.norm": vec(D, 1.0), "head": mat(config["vocab"], D)}
+    for li, layer in enumerate(config["layers"]):
+        p, m = f"l{li}.", layer["mixer"]
+        sd[p + "norm1"] = vec(D, 1.0)
+        if layer["type"] == "attention":
+            H, G, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            for n, rows in [("q", H * 2 * d)] + ([] if m.get("kv_from") is not None else [("k", G * 2 * d), ("v", G * e)]):
+                sd[p + "mix." + n] = mat(rows, D)
+                if m.get("conv"):
+                    sd[p + f"mix.{n}.conv"] = (torch.randn(rows, m["conv"], device=dev, generator=g) * 0.5).to(torch.bfloat16)
+                if n != "v":
+                    sd[p + f"mix.{n}.norm"] = vec(d, 1.0)
+            for n in ("lq1", "lk1", "lq2", "lk2"):
+                sd[p + "mix." + n] = vec(d)
+            sd[p + "mix.g"], sd[p + "mix.o"] = mat(H, D), mat(D, H * e)
+        else:
+            H, d, e = m["heads"], m["dim"], m["vdim"]
+            sd[p + "mix.q"], sd[p + "mix.f"], sd[p + "mix.v"], sd[p + "mix.o"] = mat(H * d, D), mat(H * d, D), mat(H * e, D), mat(D, H * e)
+            sd[p + "mix.f.b"] = vec(H * d, 1.0, 1.0)
+            sd[p + "mix.lower"] = torch.sigmoid(torch.randn(H * d, device=dev, generator=g)).to(torch.bfloat16)
+            sd[p + "mix.norm"] = vec(e, 1.0)
+        if layer.get("mlp") is not None:
+            ff = layer["mlp"]["ff"]
+            sd[p + "norm2"] = vec(D, 1.0)
+            sd[p + "mlp.gate"], sd[p + "mlp.up"], sd[p + "mlp.down"] = mat(ff, D), mat(ff, D), mat(D, ff)
+    return sd
+
+
+def build_random(config: dict, dtype=torch.bfloat16, device="cuda", seed: int = 0) -> RaggedDecoder:
+    return build_engine(read_config(config), random_state_dict(config, device, seed), dtype, device)
