@@ -2,6 +2,9 @@
 
   bigdl_amd/lib/libbigdl_host.so   g++  -O3 -fopenmp   (quantizers, re-layout, CPU matmul)
   bigdl_amd/lib/libbigdl_hip.so    hipcc --offload-arch=gfx950  (all device kernels + decode engine)
+  bigdl_amd/lib/libbigdl_ragged.so hipcc --offload-arch=gfx950  (csrc/ragged: the kernels of the ragged engine; a library
+                                   of its own so that a checkout without built files that only serves such a model
+                                   compiles two translation units, see ops/ragged.py::build)
 
 Both expose a plain C ABI and are loaded with ctypes, so neither needs the PyTorch
 headers: a full rebuild is a few seconds per file and hipcc cross-compiles gfx950
@@ -84,7 +87,13 @@ def build_hip(jobs=8, force=False) -> Path | None:
     return out
 
 
+def build_ragged(force=False) -> Path:
+    from ..ops import ragged
+    return ragged.build(force=force)
+
+
 def build_all(jobs=8, force=False):
+    build_ragged(force)
     return build_host(jobs, force), build_hip(jobs, force)
 
 

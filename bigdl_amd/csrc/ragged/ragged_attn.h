@@ -1,0 +1,24 @@
+// Argument block shared by the two paged attention kernels.
+#pragma once
+#include "ragged_common.h"
+
+struct AttnArgs {
+  const float* q;        // [T, H, MAPS, d]  normed and rotated
+  const void* kpages;    // [num_pages, G, PAGE, MAPS * d]
+  const void* vpages;    // [num_pages, G, PAGE, vd]
+  void* out;             // [T, H * vd]
+  const void* gate;      // gate logits: row t, column gate0 + h of a [T, ldg] matrix, or null
+  int64_t ldg;
+  int gate0;
+  int H, G, d, vd;
+  int window, keep_first;   // key j is visible from i if j <= i and (i - j < window or j < keep_first); window <= 0: all
+  float scale;
+  float lambda;          // two maps: o = a1 - lambda * a2
+  float out_scale;       // applied after the output norm
+  int out_norm;          // divide each head's output by its root mean square
+  float eps;
+  const int* rows;       // row-wise kernel: the token rows to serve (null: all T rows)
+  int n_rows;
+  const int* tiles;      // MFMA kernel: [n_tiles][2] = (sequence in the batch, first row of the tile inside its portion)
+  int n_tiles;
+};

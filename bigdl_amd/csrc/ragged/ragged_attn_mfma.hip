@@ -1,0 +1,238 @@
+// Paged attention for long bfloat16 prompt portions on the matrix cores (v_mfma_f32_16x16x32_bf16), same semantics as
+// paged_attn_kernel in ragged_attn.hip.
+//
+//  * workgroup = 64 consecutive rows of one sequence's portion and one query head; wavefront w owns rows 16 w .. 16 w + 15.
+//  * a cache page is the key tile.  Scores are computed transposed, S^T = K Q^T, so that a lane holds ONE query (its
+//    column) and 4 keys of each 16-key block: running maximum, normaliser and rescale factor are per-lane scalars
+//    (two cross-lane steps join the 4 lanes of a query), and the exponentials are already laid out as the B operand of
+//    the second product O^T += V^T P^T, with the keys of a 32-key chunk in the order (4 g + j, 16 + 4 g + j).
+//  * K fragments come straight from the page (16 bytes per lane); the value tile is transposed into LDS once per page
+//    by the whole workgroup and read back as A fragments (two 8-byte reads per fragment).
+//  * softmax weights stay 32-bit quantities: each is split into two bfloat16 terms (p = hi + lo) that go through the
+//    matrix core one after the other, so the second product loses nothing beyond the values' own 16 bits.
+//  * both maps of a differential head share the K page walk and the value tile.
+#include "ragged_attn.h"
+
+using namespace ragged;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int MF_DK = 4;     // 32-channel steps of a map: d <= 128
+constexpr int MF_NEB = 8;    // 16-channel blocks of the values: vd <= 128
+constexpr int MF_LDV = PAGE + 8;
+
+union Frag {
+  bf16x8 v;
+  uint32_t u[4];
+  uint16_t h[8];
+  uint4 q;
+  uint2 d2[2];
+};
+
+__device__ __forceinline__ uint16_t bf_bits(float f) { return from_f<bf16>(f).b; }
+
+template <int MAPS>
+__global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch bt) {
+  __shared__ __attribute__((aligned(16))) uint16_t vt[MF_NEB * 16 * MF_LDV];      // V^T [vd][PAGE (+ pad)]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int lq = lane & 15, g4 = lane >> 4;
+  const int tile = blockIdx.x / a.H, h = blockIdx.x % a.H;
+  const int b = a.tiles[2 * tile], row0 = a.tiles[2 * tile + 1];
+  const int start = bt.seq_start[b], n = bt.seq_start[b + 1] - start, past = bt.seq_past[b];
+  const int gk = h / (a.H / a.G);
+  const int qd = MAPS * a.d;
+  const int dk = (a.d + 31) / 32, neb = a.vd / 16;
+  const int nrows = n - row0 < 64 ? n - row0 : 64;          // rows of this tile
+  const int myrow = row0 + 16 * wave + lq;                  // this lane's query inside the portion
+  const bool rowok = 16 * wave + lq < nrows;
+  const int qpos = rowok ? past + myrow : -1;
+  const int64_t t = start + (rowok ? myrow : row0);
+
+  // queries as B fragments: lane = query lq, channels 32 ks + 8 g4 .. + 7
+  Frag qf[MAPS][MF_DK];
+#pragma unroll
+  for (int mp = 0; mp < MAPS; ++mp)
+#pragma unroll
+    for (int ks = 0; ks < MF_DK; ++ks) {
+      const int ch = 32 * ks + 8 * g4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) qf[mp][ks].u[e] = 0;
+      if (ks < dk && ch < a.d && rowok) {
+        const float* qp = a.q + ((t * a.H + h) * MAPS + mp) * a.d + ch;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[mp][ks].h[e] = bf_bits(qp[e]);
+      }
+    }
+
+  const int p_first = past + row0, p_last = past + row0 + nrows - 1;
+  const bool win = a.window > 0;
+  const int keep = win ? a.keep_first : 0;
+  const int lo_tile = win ? (p_first - a.window + 1 > 0 ? p_first - a.window + 1 : 0) : 0;
+  const int pl = lo_tile / PAGE, last = p_last / PAGE;
+  const int kept_pages = (keep + PAGE - 1) / PAGE < pl ? (keep + PAGE - 1) / PAGE : pl;
+  const int npg = kept_pages + last - pl + 1;
+  // what this wavefront's 16 rows can see
+  const int w_first = p_first + 16 * wave, w_last = (w_first + 15 < p_last ? w_first + 15 : p_last);
+  const int w_lo = win ? w_first - a.window + 1 : 0;
+  const bool wave_has_rows = 16 * wave < nrows;
+  const int my_lo = win ? qpos - a.window + 1 : 0;
+
+  const bf16* K = (const bf16*)a.kpages;
+  const bf16* V = (const bf16*)a.vpages;
+  const int* pages = bt.pages + (int64_t)b * bt.max_pages;
+
+  float m[MAPS], l[MAPS];
+  f32x4 O[MAPS][MF_NEB];
+#pragma unroll
+  for (int mp = 0; mp < MAPS; ++mp) {
+    m[mp] = -1e30f;
+    l[mp] = 0.f;
+#pragma unroll
+    for (int eb = 0; eb < MF_NEB; ++eb) O[mp][eb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int o = 0; o < npg; ++o) {
+    const int pg = o < kept_pages ? o : pl + (o - kept_pages);
+    const int page = pages[pg];
+    const int k0 = pg * PAGE;
+    // ---- value tile -> LDS, transposed
+    __syncthreads();                                         // the previous page's fragments have been read
+    {
+      const bf16* vsrc = V + (((int64_t)page * a.G + gk) * PAGE) * a.vd;
+      const int total = PAGE * a.vd;
+      for (int idx = threadIdx.x * 8; idx < total; idx += 256 * 8) {
+        const int key = idx / a.vd, e0 = idx % a.vd;
+        Frag f;
+        f.q = *reinterpret_cast<const uint4*>(vsrc + idx);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) vt[(e0 + u) * MF_LDV + key] = f.h[u];
+      }
+    }
+    __syncthreads();
+    const bool wave_sees = wave_has_rows && k0 <= w_last && (k0 + PAGE - 1 >= w_lo || k0 < keep);
+    if (!wave_sees) continue;
+
+    // ---- S^T = K Q^T for the 4 key blocks of the page
+    f32x4 S[MAPS][4];
+#pragma unroll
+    for (int mp = 0; mp < MAPS; ++mp)
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) S[mp][kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const bf16* kpage = K + (((int64_t)page * a.G + gk) * PAGE) * qd;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      const bf16* krow = kpage + (int64_t)(16 * kb + lq) * qd;
+#pragma unroll
+      for (int mp = 0; mp < MAPS; ++mp)
+#pragma unroll
+        for (int ks = 0; ks < MF_DK; ++ks) {
+          const int ch = 32 * ks + 8 * g4;
+          if (ks < dk) {
+            Frag kf;
+            kf.q = ch < a.d ? *reinterpret_cast<const uint4*>(krow + mp * a.d + ch) : uint4{0, 0, 0, 0};
+            S[mp][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[mp][ks].v, S[mp][kb], 0, 0, 0);
+          }
+        }
+    }
+    // ---- mask, online softmax (per-lane scalars of the lane's query), exponentials as two bfloat16 terms
+    Frag phi[MAPS][2], plo[MAPS][2];
+#pragma unroll
+    for (int mp = 0; mp < MAPS; ++mp) {
+      float mx = -1e30f;
+      bool vis[4][4];
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = k0 + 16 * kb + 4 * g4 + i;
+          vis[kb][i] = key <= qpos && (key >= my_lo || key < keep);
+          S[mp][kb][i] = vis[kb][i] ? S[mp][kb][i] * a.scale : -1e30f;
+          mx = fmaxf(mx, S[mp][kb][i]);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float mnew = fmaxf(m[mp], mx);
+      const float corr = __expf(m[mp] - mnew);
+      float sum = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float p = vis[kb][i] ? __expf(S[mp][kb][i] - mnew) : 0.f;
+          sum += p;
+          const uint16_t hi = bf_bits(p);
+          const float rest = p - __uint_as_float((uint32_t)hi << 16);
+          phi[mp][kb >> 1].h[4 * (kb & 1) + i] = hi;
+          plo[mp][kb >> 1].h[4 * (kb & 1) + i] = bf_bits(rest);
+        }
+      sum += __shfl_xor(sum, 16, 64);
+      sum += __shfl_xor(sum, 32, 64);
+      l[mp] = l[mp] * corr + sum;
+      m[mp] = mnew;
+#pragma unroll
+      for (int eb = 0; eb < MF_NEB; ++eb) O[mp][eb] *= corr;
+    }
+    // ---- O^T += V^T P^T
+#pragma unroll
+    for (int eb = 0; eb < MF_NEB; ++eb) {
+      if (eb < neb) {
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          Frag vf;
+          const uint16_t* vrow = vt + (16 * eb + lq) * MF_LDV + 32 * c + 4 * g4;
+          vf.d2[0] = *reinterpret_cast<const uint2*>(vrow);
+          vf.d2[1] = *reinterpret_cast<const uint2*>(vrow + 16);
+#pragma unroll
+          for (int mp = 0; mp < MAPS; ++mp) {
+            O[mp][eb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, phi[mp][c].v, O[mp][eb], 0, 0, 0);
+            O[mp][eb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, plo[mp][c].v, O[mp][eb], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+  if (!rowok) return;
+  // ---- epilogue: combine the maps, per-head norm, gate; the lane holds channels 16 eb + 4 g4 + i of its query
+  const float c0 = 1.0f / l[0];
+  const float c1 = MAPS == 2 ? a.lambda / l[MAPS - 1] : 0.f;
+  float ss = 0.f;
+#pragma unroll
+  for (int eb = 0; eb < MF_NEB; ++eb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float v = O[0][eb][i] * c0;
+      if (MAPS == 2) v -= O[MAPS - 1][eb][i] * c1;
+      if (eb >= neb) v = 0.f;
+      O[0][eb][i] = v;
+      ss += v * v;
+    }
+  ss += __shfl_xor(ss, 16, 64);
+  ss += __shfl_xor(ss, 32, 64);
+  float f = a.out_scale;
+  if (a.out_norm) f *= 1.0f / sqrtf(ss / (float)a.vd + a.eps);
+  if (a.gate) f *= sigmoidf_(to_f(((const bf16*)a.gate)[t * a.ldg + a.gate0 + h]));
+  uint16_t* orow = (uint16_t*)a.out + t * (int64_t)(a.H * a.vd) + (int64_t)h * a.vd;
+#pragma unroll
+  for (int eb = 0; eb < MF_NEB; ++eb)
+    if (eb < neb) {
+      uint2 w;
+      w.x = (uint32_t)bf_bits(O[0][eb][0] * f) | ((uint32_t)bf_bits(O[0][eb][1] * f) << 16);
+      w.y = (uint32_t)bf_bits(O[0][eb][2] * f) | ((uint32_t)bf_bits(O[0][eb][3] * f) << 16);
+      *reinterpret_cast<uint2*>(orow + 16 * eb + 4 * g4) = w;
+    }
+}
+
+// 1 when the MFMA kernel serves this head layout (bfloat16 only)
+extern "C" int ragged_paged_attn_mfma_ok(int d, int vd) {
+  return d % 8 == 0 && d <= 32 * MF_DK && vd % 16 == 0 && vd <= 16 * MF_NEB;
+}
+
+extern "C" int ragged_paged_attn_mfma(AttnArgs a, Batch bt, int maps, hipStream_t st) {
+  if (bt.T <= 0 || a.H <= 0 || a.G <= 0 || a.H % a.G || !ragged_paged_attn_mfma_ok(a.d, a.vd)) return -1;
+  if ((maps != 1 && maps != 2) || !a.tiles || a.n_tiles <= 0 || (int64_t)a.n_tiles * a.H > 0x7fffffff) return -1;
+  const unsigned grid = (unsigned)(a.n_tiles * a.H);
+  if (maps == 2) hipLaunchKernelGGL((paged_attn_mfma_kernel<2>), dim3(grid), dim3(256), 0, st, a, bt);
+  else hipLaunchKernelGGL((paged_attn_mfma_kernel<1>), dim3(grid), dim3(256), 0, st, a, bt);
+  return RAGGED_LAUNCH_OK();
+}

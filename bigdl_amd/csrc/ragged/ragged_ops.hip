@@ -249,23 +249,36 @@ __global__ __launch_bounds__(64) void hgrn2_scan_kernel(const float* __restrict_
     S[k] = (past > 0 && colok && k < DR && row < d) ? sp[(int64_t)row * vd + col] : 0.f;
   }
   const int HD = H * d;
-  for (int i = 0; i < n; ++i) {
+  // the loads of token i + 1 are issued before the arithmetic of token i: a step otherwise waits a memory round trip
+  float qn[HG_DR], fn[HG_DR], vn = 0.f;
+  auto fetch = [&](int i) {
     const int64_t t = start + i;
     const float* qrow = qf + t * HD + h * d;
     const float* frow = ff + t * HD + h * d;
-    const float v = colok ? to_f(P[t * ldp + v0 + h * vd + col]) : 0.f;
-    float acc = 0.f;
 #pragma unroll
     for (int k = 0; k < HG_DR; ++k) {
       const int row = row0 + k;
-      if (k < DR && row < d) {
-        const float f = frow[row];
-        S[k] = f * S[k] + (1.0f - f) * v;
-        acc += S[k] * qrow[row];
-      }
+      const bool ok = k < DR && row < d;
+      qn[k] = ok ? qrow[row] : 0.f;
+      fn[k] = ok ? frow[row] : 1.f;
+    }
+    vn = colok ? to_f(P[t * ldp + v0 + h * vd + col]) : 0.f;
+  };
+  if (n > 0) fetch(0);
+  for (int i = 0; i < n; ++i) {
+    float qc[HG_DR], fc[HG_DR];
+#pragma unroll
+    for (int k = 0; k < HG_DR; ++k) { qc[k] = qn[k]; fc[k] = fn[k]; }
+    const float v = vn;
+    if (i + 1 < n) fetch(i + 1);
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < HG_DR; ++k) {
+      S[k] = fc[k] * S[k] + (1.0f - fc[k]) * v;
+      acc += S[k] * qc[k];
     }
     for (int o = 1; o < R; o <<= 1) acc += __shfl_xor(acc, o, 64);
-    if (r == 0 && colok) out[t * (int64_t)(H * vd) + h * vd + col] = acc;
+    if (r == 0 && colok) out[(int64_t)(start + i) * (H * vd) + h * vd + col] = acc;
   }
 #pragma unroll
   for (int k = 0; k < HG_DR; ++k) {

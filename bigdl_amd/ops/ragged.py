@@ -71,7 +71,8 @@ class _AttnArgs(ctypes.Structure):
                 ("gate", ctypes.c_void_p), ("ldg", ctypes.c_int64), ("gate0", ctypes.c_int), ("H", ctypes.c_int),
                 ("G", ctypes.c_int), ("d", ctypes.c_int), ("vd", ctypes.c_int), ("window", ctypes.c_int),
                 ("keep_first", ctypes.c_int), ("scale", ctypes.c_float), ("lam", ctypes.c_float),
-                ("out_scale", ctypes.c_float), ("out_norm", ctypes.c_int), ("eps", ctypes.c_float)]
+                ("out_scale", ctypes.c_float), ("out_norm", ctypes.c_int), ("eps", ctypes.c_float),
+                ("rows", ctypes.c_void_p), ("n_rows", ctypes.c_int), ("tiles", ctypes.c_void_p), ("n_tiles", ctypes.c_int)]
 
 
 def lib():
@@ -89,6 +90,8 @@ def lib():
         L.ragged_hgrn2_scan.argtypes = [vp, vp, vp, i64, ci, vp, vp, ci, ci, ci, _Batch, ci, vp]
         L.ragged_row_norm.argtypes = [vp, vp, vp, i64, ci, cf, ci, vp]
         L.ragged_paged_attn.argtypes = [_AttnArgs, _Batch, ci, ci, vp]
+        L.ragged_paged_attn_mfma.argtypes = [_AttnArgs, _Batch, ci, vp]
+        L.ragged_paged_attn_mfma_ok.argtypes = [ci, ci]
         _LIB = L
     return _LIB
 
@@ -121,6 +124,23 @@ class BatchMeta:
         self.seq_start, self.seq_past, self.seq_slot = buf[o[2]:o[3]], buf[o[3]:o[4]], buf[o[4]:o[5]]
         self.pages = buf[o[5]:].view(B, self.max_pages)
         self._c = None
+        self._split = {}
+
+    def attn_split(self, min_rows: int):
+        """Portions of at least ``min_rows`` rows as 64-row tiles [(sequence, first row)] for the matrix-core attention
+        kernel, all other token rows as a list for the row-wise kernel: (tiles, n_tiles, rows, n_rows), device int32."""
+        if min_rows not in self._split:
+            tiles, rows = [], []
+            for b, (_, _, n, _) in enumerate(self.seqs):
+                if n >= min_rows:
+                    tiles += [v for r0 in range(0, n, 64) for v in (b, r0)]
+                else:
+                    rows += range(self.start[b], self.start[b] + n)
+            buf = torch.tensor(tiles + rows + [0], dtype=torch.int32)
+            if self.buf.device.type == "cuda":
+                buf = buf.pin_memory().to(self.buf.device, non_blocking=True)
+            self._split[min_rows] = (buf[:len(tiles)], len(tiles) // 2, buf[len(tiles):len(tiles) + len(rows)], len(rows))
+        return self._split[min_rows]
 
     def c(self):
         if self._c is None:
@@ -163,6 +183,8 @@ def _page_check(meta: BatchMeta, pages: torch.Tensor):
 class HipOps:
     """The kernels.  Every call checks shapes against what the kernel's indexing assumes before it launches."""
     name = "hip"
+    mfma = os.environ.get("BIGDL_RAGGED_MFMA", "1") != "0"      # 0: every row through the row-wise attention kernel
+    mfma_min_rows = 8
 
     def sum_group_norm(self, x, y, w, groups, alpha, eps, act, x_out=None, want_act=True):
         _f32(x, w, x_out)
@@ -285,6 +307,16 @@ class HipOps:
             a.gate, a.ldg, a.gate0 = gate.data_ptr(), gate.stride(0), gate0
         a.H, a.G, a.d, a.vd, a.window, a.keep_first = H, G, d, vd, window, keep_first
         a.scale, a.lam, a.out_scale, a.out_norm, a.eps = scale, lam, out_scale, int(out_norm), eps
+        if kpages.dtype == torch.bfloat16 and self.mfma and lib().ragged_paged_attn_mfma_ok(d, vd):
+            # long portions on the matrix cores, single tokens and short portions row by row
+            tiles, n_tiles, rows, n_rows = meta.attn_split(self.mfma_min_rows)
+            if n_tiles:
+                a.tiles, a.n_tiles = tiles.data_ptr(), n_tiles
+                _ok(lib().ragged_paged_attn_mfma(a, meta.c(), maps, _stream()), "paged_attn_mfma")
+            if n_rows:
+                a.rows, a.n_rows = rows.data_ptr(), n_rows
+                _ok(lib().ragged_paged_attn(a, meta.c(), maps, _DT[kpages.dtype], _stream()), "paged_attn")
+            return out
         _ok(lib().ragged_paged_attn(a, meta.c(), maps, _DT[kpages.dtype], _stream()), "paged_attn")
         return out
 

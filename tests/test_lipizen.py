@@ -408,3 +408,47 @@ def test_trace_runner_replays_steps(tmp_path):
     close(got1, want[[2]])
     got2 = torch.from_numpy(np.fromfile(os.path.join(out, "2.f32"), dtype="<f4")).view(1, -1).double()
     close(got2, want[[19]])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,d,e,window,keep", [(4, 2, 64, 128, 100, 5), (2, 2, 48, 96, 70, 0), (3, 1, 16, 32, 0, 0),
+                                                 (2, 1, 128, 64, 300, 70), (2, 2, 40, 16, 64, 64)])
+def test_matrix_core_attention_against_the_plain_statement(H, G, d, e, window, keep):
+    """bfloat16 prompt portions take the MFMA kernel, single tokens the row-wise one: both against float64 attention
+    over the same (bfloat16-rounded) queries, keys and values, in portions that cut pages and windows."""
+    g = torch.Generator().manual_seed(91)
+    T = 333
+    bf = lambda x: x.to(torch.bfloat16).to(O.F64)                                   # noqa: E731
+    q = bf(torch.randn(T, H, 2, d, generator=g, dtype=O.F64))
+    k = bf(torch.randn(T, G, 2, d, generator=g, dtype=O.F64))
+    v = bf(torch.randn(T, G, e, generator=g, dtype=O.F64))
+    scale, lam = d ** -0.5 * 2.0, 0.6
+    want = torch.zeros(T, H, e, dtype=O.F64)
+    for i in range(T):
+        js = [x for x in range(T) if O.sees(i, x, window or None, keep)]
+        for hh in range(H):
+            kk = hh // (H // G)
+            want[i, hh] = O.softmax_attend(q[i, hh, 0], k[js, kk, 0], v[js, kk], scale) - \
+                lam * O.softmax_attend(q[i, hh, 1], k[js, kk, 1], v[js, kk], scale)
+    device = "cuda"
+    ops = R.ops_for(device)
+    pool = PagedStatePool({0: [("kv", G, 2 * d, e)]}, 64 * 8, 2, torch.bfloat16, device)
+    pool.free_pages = [3, 0, 7, 5, 1, 6, 2, 4]
+    slot = pool.admit()
+    got, at = [], 0
+    for n in (70, 9, 1, 130, 64, 8, 1, 50):
+        meta = _meta_for(pool, slot, n, device)
+        for i in range(n):
+            pos = at + i
+            pg = pool.pages_of[slot][pos // 64]
+            pool.k[0][pg, :, pos % 64] = k[pos].reshape(G, 2 * d).to(device, torch.bfloat16)
+            pool.v[0][pg, :, pos % 64] = v[pos].to(device, torch.bfloat16)
+        qq = q[at:at + n].reshape(n, H * 2 * d).float().to(device).contiguous()
+        got.append(ops.paged_attn(qq, pool.k[0], pool.v[0], meta, maps=2, H=H, G=G, d=d, vd=e, window=window,
+                                  keep_first=keep, scale=scale, lam=lam, out_scale=1.0, out_norm=False, eps=1e-6))
+        pool.commit(slot, n)
+        at += n
+    assert at == T
+    got = torch.cat(got).double().cpu().view(T, H, e)
+    # the output is rounded to bfloat16 (2^-9 relative); the 32-bit softmax weights add nothing visible to that
+    assert float((got - want).abs().max()) < 0.02 * float(want.abs().max()), float((got - want).abs().max())
