@@ -26,15 +26,34 @@ template <> __device__ __forceinline__ bf16 from_f<bf16>(float f) {
   return r;
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+// Cross-lane steps inside a row of 16 lanes are DPP moves (a few cycles); only the two steps across rows go through
+// the LDS crossbar.  DPP controls: 0xB1 / 0x4E swap lanes inside a quad (xor 1 / xor 2), 0x141 mirrors 8 lanes,
+// 0x140 mirrors 16: for a sum or a maximum over a whole group a mirror serves as well as an xor.
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+// sum over groups of R neighbouring lanes (R a power of two), result in every lane of the group
+__device__ __forceinline__ float group_sum(float v, int R) {
+  if (R >= 2) v += dpp_move<0xB1>(v);
+  if (R >= 4) v += dpp_move<0x4E>(v);
+  if (R >= 8) v += dpp_move<0x141>(v);
+  if (R >= 16) v += dpp_move<0x140>(v);
+  if (R >= 32) v += __shfl_xor(v, 16, 64);
+  if (R >= 64) v += __shfl_xor(v, 32, 64);
   return v;
 }
+__device__ __forceinline__ float wave_sum(float v) { return group_sum(v, 64); }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
+  v = fmaxf(v, dpp_move<0xB1>(v));
+  v = fmaxf(v, dpp_move<0x4E>(v));
+  v = fmaxf(v, dpp_move<0x141>(v));
+  v = fmaxf(v, dpp_move<0x140>(v));
+  v = fmaxf(v, __shfl_xor(v, 16, 64));
+  return fmaxf(v, __shfl_xor(v, 32, 64));
+}
+// the value of lane `j` (the same j in every lane) in all lanes: v_readlane, no trip through LDS
+__device__ __forceinline__ float lane_value(float v, int j) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), j));
 }
 
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }

@@ -45,7 +45,8 @@ extern "C" int ragged_sum_group_norm(const float* x, const void* y, const float*
 // ---------------------------------------------------------------------------------------------------------------
 // Short causal convolution over time per channel, then (optionally) RMS norm over groups of `gsize` channels with a
 // weight shared by all groups, then (optionally) rotation of the first `rot` channels of each group (pairs i, i + rot/2,
-// angle = position * inv_freq[i]), then a store into a dense float buffer or into cache pages.
+// cosine and sine of the row's angles from a table made once per step), then a store into a dense float buffer or into
+// cache pages.
 struct ConvHeadArgs {
   const void* P;          // [T, ldp] projections of this step
   int64_t ldp;
@@ -57,7 +58,7 @@ struct ConvHeadArgs {
   const float* normw;     // [gsize] or null
   float eps;
   int rot;                // 0: no rotation
-  const float* inv_freq;  // [rot / 2]
+  const float* cossin;    // [T, rot / 2, 2]: cos and sin of position * frequency for every row of the batch
   float* out_dense;       // [T, ngroups * gsize] or null
   void* pages;            // [num_pages, heads, PAGE, rowlen]
   int rowlen, heads;
@@ -116,9 +117,8 @@ __global__ __launch_bounds__(256) void conv_head_kernel(ConvHeadArgs a, Batch bt
     float v = buf[c];
     if (c < a.rot) {
       const int i = c < half ? c : c - half;
-      const float ang = (float)pos * a.inv_freq[i];
-      float sn, cs;
-      sincosf(ang, &sn, &cs);
+      const float2 tr = *reinterpret_cast<const float2*>(a.cossin + ((int64_t)t * half + i) * 2);
+      const float cs = tr.x, sn = tr.y;
       v = c < half ? buf[c] * cs - buf[c + half] * sn : buf[c] * cs + buf[c - half] * sn;
     }
     const int f = grp * a.gsize + c;
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256) void conv_head_kernel(ConvHeadArgs a, Batch bt
 extern "C" int ragged_conv_head(ConvHeadArgs a, Batch bt, int dtype, hipStream_t st) {
   if (bt.T <= 0 || a.ngroups <= 0 || a.gsize <= 0 || a.gsize > 2048) return -1;
   if (a.cw && (a.taps < 1 || a.taps > 16 || (a.taps > 1 && !a.state))) return -1;
-  if (a.rot < 0 || (a.rot & 1) || a.rot > a.gsize || (a.rot && !a.inv_freq)) return -1;
+  if (a.rot < 0 || (a.rot & 1) || a.rot > a.gsize || (a.rot && !a.cossin)) return -1;
   if (!a.out_dense && (!a.pages || a.rowlen <= 0 || (a.ngroups * a.gsize) % a.rowlen || a.heads * a.rowlen != a.ngroups * a.gsize))
     return -1;
   const int64_t items = (int64_t)bt.T * a.ngroups;
@@ -227,63 +227,120 @@ extern "C" int ragged_hgrn2_gates(const void* P, int64_t ldp, int q0, int f0, co
 }
 
 // Scan: per head S <- diag(f_t) S + (1 - f_t) v_t^T, o_t = S^T q_t, S float [d, vd] per (slot, head).
-// A wavefront owns 64 / R columns of S; R neighbouring lanes share a column and hold DR = ceil(d / R) <= 32 of its rows
-// in registers.  The wavefront walks the tokens of its sequence in order with no barrier: the only cross-lane step is
-// the sum of R partial dot products.  Grid: (column blocks, heads, sequences).
+// A wavefront owns 64 / R columns of S; R neighbouring lanes share a column, lane r of them holds rows 32 r .. 32 r + 31
+// in registers (R = d / 32 rounded up to a power of two; rows past d carry q = 0, f = 1 and stay zero), so the only
+// cross-lane step of a token is the sum of R partial dot products (DPP moves).  A workgroup is four such wavefronts.
+// Gates and queries of a block of TB tokens are brought into LDS by the whole workgroup with coalesced loads while the
+// previous block is being scanned (register look-ahead, two LDS buffers); a step reads its 32 gates and 32 queries
+// back as 16-byte broadcasts with no condition around them, so all reads of a step are in flight together.
+// Grid: (column blocks, heads, sequences).
 constexpr int HG_DR = 32;
+constexpr int HG_SEG = HG_DR + 4;   // LDS floats per lane group and token (padding shifts the banks between groups)
+constexpr int HG_TBR = 64;          // TB * R <= this
+constexpr int HG_PRE = 2 * HG_TBR * HG_DR / 256;
 
 template <typename T>
-__global__ __launch_bounds__(64) void hgrn2_scan_kernel(const float* __restrict__ qf, const float* __restrict__ ff,
-                                                        const T* __restrict__ P, int64_t ldp, int v0, float* __restrict__ state,
-                                                        float* __restrict__ out, int H, int d, int vd, int R, int DR, Batch bt) {
-  const int b = blockIdx.z, h = blockIdx.y, lane = threadIdx.x;
-  const int r = lane % R, col = blockIdx.x * (64 / R) + lane / R;
+__global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* __restrict__ qf, const float* __restrict__ ff,
+                                                         const T* __restrict__ P, int64_t ldp, int v0, float* __restrict__ state,
+                                                         float* __restrict__ out, int H, int d, int vd, int R, int TB, Batch bt) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];   // 2 x { q[TB][R][SEG], f[TB][R][SEG], v[TB][wcols] }
+  const int b = blockIdx.z, h = blockIdx.y, tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int cols = 64 / R, wcols = 4 * cols;
+  const int r = lane % R, lc = wave * cols + lane / R;     // column inside the workgroup's block
+  const int col = blockIdx.x * wcols + lc;
   const int start = bt.seq_start[b], n = bt.seq_start[b + 1] - start, past = bt.seq_past[b], slot = bt.seq_slot[b];
   const bool colok = col < vd;
-  const int row0 = r * DR;
+  const int row0 = r * HG_DR;
+  const int HD = H * d;
+  const int qsz = TB * R * HG_SEG;                         // floats of q (and of f) in a buffer
+  const int bufsz = 2 * qsz + TB * wcols;
   float S[HG_DR];
   float* sp = state + (((int64_t)slot * H + h) * d) * vd;
-#pragma unroll
-  for (int k = 0; k < HG_DR; ++k) {
-    const int row = row0 + k;
-    S[k] = (past > 0 && colok && k < DR && row < d) ? sp[(int64_t)row * vd + col] : 0.f;
-  }
-  const int HD = H * d;
-  // the loads of token i + 1 are issued before the arithmetic of token i: a step otherwise waits a memory round trip
-  float qn[HG_DR], fn[HG_DR], vn = 0.f;
-  auto fetch = [&](int i) {
-    const int64_t t = start + i;
-    const float* qrow = qf + t * HD + h * d;
-    const float* frow = ff + t * HD + h * d;
+  {
+    const int cc = colok ? col : vd - 1;
 #pragma unroll
     for (int k = 0; k < HG_DR; ++k) {
       const int row = row0 + k;
-      const bool ok = k < DR && row < d;
-      qn[k] = ok ? qrow[row] : 0.f;
-      fn[k] = ok ? frow[row] : 1.f;
+      const float v = sp[(int64_t)(row < d ? row : d - 1) * vd + cc];    // no condition around the load
+      S[k] = (past > 0 && colok && row < d) ? v : 0.f;
     }
-    vn = colok ? to_f(P[t * ldp + v0 + h * vd + col]) : 0.f;
+  }
+  float pre[HG_PRE], prev[4];
+  const int nel = TB * R * HG_DR;                          // q (or f) elements of a block, padded rows included
+  auto fetch = [&](int i0) {                               // block of tokens i0 .. i0 + TB - 1 into registers
+#pragma unroll
+    for (int u = 0; u < HG_PRE; ++u) {
+      const int e = tid + 256 * u;
+      const int which = e >= nel, rem = which ? e - nel : e;
+      const int tk = rem / (R * HG_DR), row = rem % (R * HG_DR);
+      float v = which ? 1.f : 0.f;                         // padding: f = 1, q = 0
+      if (e < 2 * nel && row < d && i0 + tk < n) v = (which ? ff : qf)[(int64_t)(start + i0 + tk) * HD + h * d + row];
+      pre[u] = v;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = tid + 256 * u;
+      float v = 0.f;
+      if (e < TB * wcols) {
+        const int tk = e / wcols, c = blockIdx.x * wcols + e % wcols;
+        if (i0 + tk < n && c < vd) v = to_f(P[(int64_t)(start + i0 + tk) * ldp + v0 + h * vd + c]);
+      }
+      prev[u] = v;
+    }
   };
-  if (n > 0) fetch(0);
-  for (int i = 0; i < n; ++i) {
-    float qc[HG_DR], fc[HG_DR];
+  auto stash = [&](float* buf) {
 #pragma unroll
-    for (int k = 0; k < HG_DR; ++k) { qc[k] = qn[k]; fc[k] = fn[k]; }
-    const float v = vn;
-    if (i + 1 < n) fetch(i + 1);
-    float acc = 0.f;
-#pragma unroll
-    for (int k = 0; k < HG_DR; ++k) {
-      S[k] = fc[k] * S[k] + (1.0f - fc[k]) * v;
-      acc += S[k] * qc[k];
+    for (int u = 0; u < HG_PRE; ++u) {
+      const int e = tid + 256 * u;
+      if (e < 2 * nel) {
+        const int which = e >= nel, rem = which ? e - nel : e;
+        const int tk = rem / (R * HG_DR), row = rem % (R * HG_DR);
+        buf[which * qsz + (tk * R + row / HG_DR) * HG_SEG + row % HG_DR] = pre[u];
+      }
     }
-    for (int o = 1; o < R; o <<= 1) acc += __shfl_xor(acc, o, 64);
-    if (r == 0 && colok) out[(int64_t)(start + i) * (H * vd) + h * vd + col] = acc;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = tid + 256 * u;
+      if (e < TB * wcols) buf[2 * qsz + e] = prev[u];
+    }
+  };
+  if (n > 0) { fetch(0); stash(smem); }
+  __syncthreads();
+  int cur = 0;
+  for (int i0 = 0; i0 < n; i0 += TB) {
+    const bool more = i0 + TB < n;
+    if (more) fetch(i0 + TB);
+    const float* buf = smem + cur * bufsz;
+    const int nt = n - i0 < TB ? n - i0 : TB;
+    for (int tk = 0; tk < nt; ++tk) {
+      const float4* q4 = reinterpret_cast<const float4*>(buf + (tk * R + r) * HG_SEG);
+      const float4* f4 = reinterpret_cast<const float4*>(buf + qsz + (tk * R + r) * HG_SEG);
+      float qv[HG_DR], fv[HG_DR];
+#pragma unroll
+      for (int k = 0; k < HG_DR / 4; ++k) {
+        const float4 a = q4[k], c = f4[k];
+        qv[4 * k] = a.x; qv[4 * k + 1] = a.y; qv[4 * k + 2] = a.z; qv[4 * k + 3] = a.w;
+        fv[4 * k] = c.x; fv[4 * k + 1] = c.y; fv[4 * k + 2] = c.z; fv[4 * k + 3] = c.w;
+      }
+      const float v = buf[2 * qsz + tk * wcols + lc];
+      float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k = 0; k < HG_DR; ++k) {
+        S[k] = fv[k] * S[k] + (1.0f - fv[k]) * v;
+        acc[k & 3] += S[k] * qv[k];
+      }
+      const float tot = group_sum((acc[0] + acc[1]) + (acc[2] + acc[3]), R);
+      if (r == 0 && colok) out[(int64_t)(start + i0 + tk) * (H * vd) + h * vd + col] = tot;
+    }
+    if (more) stash(smem + (cur ^ 1) * bufsz);
+    __syncthreads();
+    cur ^= 1;
   }
 #pragma unroll
   for (int k = 0; k < HG_DR; ++k) {
     const int row = row0 + k;
-    if (colok && k < DR && row < d) sp[(int64_t)row * vd + col] = S[k];
+    if (colok && row < d) sp[(int64_t)row * vd + col] = S[k];
   }
 }
 
@@ -292,9 +349,12 @@ extern "C" int ragged_hgrn2_scan(const float* qf, const float* ff, const void* P
   if (bt.B <= 0 || H <= 0 || d <= 0 || vd <= 0 || d > HG_DR * 64) return -1;
   int R = 1;
   while (R * HG_DR < d) R <<= 1;
-  const int DR = (d + R - 1) / R, cols = 64 / R;
-  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((hgrn2_scan_kernel<T>), dim3((vd + cols - 1) / cols, H, bt.B), dim3(64), 0, st, qf, ff,
-                                            (const T*)P, ldp, v0, state, out, H, d, vd, R, DR, bt))
+  const int wcols = 4 * (64 / R);
+  int TB = HG_TBR / R < 16 ? HG_TBR / R : 16;
+  if (TB * wcols > 4 * 256) TB = 4 * 256 / wcols;           // the value look-ahead holds 4 floats per thread
+  const size_t sm = 2 * (size_t)(2 * TB * R * HG_SEG + TB * wcols) * sizeof(float);
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((hgrn2_scan_kernel<T>), dim3((vd + wcols - 1) / wcols, H, bt.B), dim3(256), sm, st, qf,
+                                            ff, (const T*)P, ldp, v0, state, out, H, d, vd, R, TB, bt))
   return RAGGED_LAUNCH_OK();
 }
 

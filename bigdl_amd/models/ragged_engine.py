@@ -16,6 +16,7 @@ into arbitrary portions next to single decoded tokens run here instead:
 from __future__ import annotations
 
 import math
+import os
 import time
 from dataclasses import dataclass, field
 from typing import List, Optional, Sequence
@@ -121,6 +122,11 @@ class RaggedDecoder:
                     raise ValueError(f"layer {li}: kv_from must name an earlier attention layer with keys of its own and "
                                      "the same head layout")
         self.first_cost = self.rest_cost_mean = self.peak_memory = 0.0
+        # steps that carry one token per sequence are recorded once per (sequences, page-table width) and replayed as
+        # one hipGraph; BIGDL_RAGGED_GRAPH=0 issues them kernel by kernel like every other step
+        self.use_graph = self.device.type == "cuda" and os.environ.get("BIGDL_RAGGED_GRAPH", "1") != "0"
+        self._graphs = {}
+        self.graph_replays = 0
 
     # ------------------------------------------------------------------ state
     def state_specs(self):
@@ -148,6 +154,7 @@ class RaggedDecoder:
         p = self.pool
         if p is None or p.num_pages * R.PAGE < max_tokens or p.slots < slots or p.len_of:
             self.pool = PagedStatePool(self.state_specs(), max_tokens, slots, self.act, self.device)
+            self._graphs.clear()              # recorded steps hold the old pool's addresses
         return self.pool
 
     # ------------------------------------------------------------------ layers
@@ -187,17 +194,62 @@ class RaggedDecoder:
         """``entries``: [(slot, token ids)] with slots from ``pool.admit()``; every entry continues its sequence by
         these tokens.  ``want[i]``: indices into entry i's tokens whose logits are returned (default: the last one).
         Returns float32 logits [wanted rows, vocab] in the order of entries and indices."""
-        cfg, ops, pool = self.cfg, self.ops, self.pool
+        pool = self.pool
         seqs, ids = [], []
         for slot, toks in entries:
             if len(toks) == 0:
                 raise ValueError("an entry without tokens")
             seqs.append((slot, pool.len_of[slot], len(toks), list(pool.reserve(slot, len(toks)))))
             ids += list(toks)
-        meta = R.BatchMeta(seqs, self.device)
+        rows, at = [], 0
+        for b, (_, _, n, _) in enumerate(seqs):
+            idx = [n - 1] if want is None else want[b]
+            if any(not 0 <= i < n for i in idx):
+                raise ValueError("a wanted index outside its entry")
+            rows += [at + i for i in idx]
+            at += n
         idt = torch.tensor(ids, dtype=torch.int64)
-        if self.device.type == "cuda":
-            idt = idt.pin_memory().to(self.device, non_blocking=True)
+        if self.use_graph and collect is None and len(ids) == len(seqs) and rows == list(range(len(seqs))):
+            logits = self._decode_step(seqs, idt)
+        else:
+            if self.device.type == "cuda":
+                idt = idt.pin_memory().to(self.device, non_blocking=True)
+            logits = self._forward(R.BatchMeta(seqs, self.device), idt, rows, collect)
+        for slot, _, n, _ in seqs:
+            pool.commit(slot, n)
+        return logits
+
+    def _decode_step(self, seqs, idt):
+        """One token per sequence.  The first step of a shape runs kernel by kernel (and loads whatever is loaded
+        lazily); the second is recorded -- recording executes nothing, so cache and state are touched once per step --
+        and from then on a step is: refill the static batch description and token ids, replay."""
+        B = len(seqs)
+        width = 1
+        while width < max(len(pg) for *_, pg in seqs):
+            width *= 2
+        ent = self._graphs.get((B, width))
+        if ent is None:
+            self._graphs[(B, width)] = {}
+            return self._forward(R.BatchMeta(seqs, self.device), idt.pin_memory().to(self.device, non_blocking=True),
+                                 list(range(B)), None)
+        if not ent:
+            ent["meta"] = R.BatchMeta(seqs, self.device, max_pages=width, static=True)
+            ent["host_ids"] = torch.empty(B, dtype=torch.int64, pin_memory=True)
+            ent["ids"] = torch.zeros(B, dtype=torch.int64, device=self.device)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                ent["logits"] = self._forward(ent["meta"], ent["ids"], list(range(B)), None)
+            ent["graph"] = graph
+        ent["meta"].update(seqs)
+        ent["host_ids"].copy_(idt)
+        ent["ids"].copy_(ent["host_ids"], non_blocking=True)
+        ent["graph"].replay()
+        self.graph_replays += 1
+        return ent["logits"].clone()
+
+    def _forward(self, meta, idt, rows, collect):
+        cfg, ops = self.cfg, self.ops
         x = F.embedding(idt, self.embed).float()
         xa = x.to(self.act)
         for li, (m, mlp, lt) in enumerate(zip(cfg.mixers, cfg.mlps, self.layers)):
@@ -210,18 +262,14 @@ class RaggedDecoder:
                                         self.act)
             if collect is not None:
                 collect.append(x.clone())
-        for slot, _, n, _ in seqs:
-            pool.commit(slot, n)
-        rows = []
-        for b, (_, _, n, _) in enumerate(seqs):
-            idx = [n - 1] if want is None else want[b]
-            if any(not 0 <= i < n for i in idx):
-                raise ValueError("a wanted index outside its entry")
-            rows += [meta.start[b] + i for i in idx]
         if not rows:
             return torch.empty(0, cfg.vocab, dtype=torch.float32, device=self.device)
-        xr = x[torch.tensor(rows, dtype=torch.int64, device=self.device)].contiguous()
-        xa = ops.sum_group_norm(xr, None, self.final_norm, cfg.norm_groups, 1.0, cfg.norm_eps, self.act)
+        if rows == list(range(meta.T)):
+            xr = x                                # (the final norm writes its own output)
+        else:
+            xr = x[torch.tensor(rows, dtype=torch.int64, device=self.device)].contiguous()
+        xo = torch.empty_like(xr)
+        xa = ops.sum_group_norm(xr, None, self.final_norm, cfg.norm_groups, 1.0, cfg.norm_eps, self.act, x_out=xo)
         logits = F.linear(xa, self.head).float()
         if cfg.logit_softcap > 0:
             logits = torch.tanh(logits / cfg.logit_softcap) * cfg.logit_softcap

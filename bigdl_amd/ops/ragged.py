@@ -62,7 +62,7 @@ class _ConvHeadArgs(ctypes.Structure):
     _fields_ = [("P", ctypes.c_void_p), ("ldp", ctypes.c_int64), ("col0", ctypes.c_int), ("cw", ctypes.c_void_p),
                 ("taps", ctypes.c_int), ("C", ctypes.c_int), ("ch0", ctypes.c_int), ("state", ctypes.c_void_p),
                 ("ngroups", ctypes.c_int), ("gsize", ctypes.c_int), ("normw", ctypes.c_void_p), ("eps", ctypes.c_float),
-                ("rot", ctypes.c_int), ("inv_freq", ctypes.c_void_p), ("out_dense", ctypes.c_void_p),
+                ("rot", ctypes.c_int), ("cossin", ctypes.c_void_p), ("out_dense", ctypes.c_void_p),
                 ("pages", ctypes.c_void_p), ("rowlen", ctypes.c_int), ("heads", ctypes.c_int)]
 
 
@@ -99,14 +99,33 @@ def lib():
 class BatchMeta:
     """One step's batch: ``seqs`` is a list of (slot, past, n_new, page ids covering past + n_new tokens)."""
 
-    def __init__(self, seqs, device):
-        self.seqs = seqs
+    def __init__(self, seqs, device, max_pages=None, static=False):
+        """``static``: the device buffer keeps its address and layout (``max_pages`` fixed) and ``update`` refills it, so
+        that a step recorded into a hipGraph reads the next step's batch from the same place."""
+        device = torch.device(device)
+        self.device = device
         self.B = len(seqs)
+        self.T = sum(n for _, _, n, _ in seqs)
+        self.max_pages = max_pages or max(1, max(len(pg) for *_, pg in seqs))
+        T, B = self.T, self.B
+        size = 2 * T + 3 * B + 1 + B * self.max_pages
+        self._host = torch.empty(size, dtype=torch.int32, pin_memory=device.type == "cuda")
+        self.buf = torch.empty(size, dtype=torch.int32, device=device) if static or device.type == "cuda" else self._host
+        o = [0, T, 2 * T, 2 * T + B + 1, 2 * T + 2 * B + 1, 2 * T + 3 * B + 1]
+        buf = self.buf
+        self.tok_seq, self.tok_pos = buf[o[0]:o[1]], buf[o[1]:o[2]]
+        self.seq_start, self.seq_past, self.seq_slot = buf[o[2]:o[3]], buf[o[3]:o[4]], buf[o[4]:o[5]]
+        self.pages = buf[o[5]:].view(B, self.max_pages)
+        self.update(seqs)
+
+    def update(self, seqs):
+        """Fill the buffer for this step's sequences (same count and row total as at construction)."""
+        self.seqs = seqs
         self.start = [0]
         for _, _, n, _ in seqs:
             self.start.append(self.start[-1] + n)
-        self.T = self.start[-1]
-        self.max_pages = max(1, max(len(pg) for *_, pg in seqs))
+        if len(seqs) != self.B or self.start[-1] != self.T or max(len(pg) for *_, pg in seqs) > self.max_pages:
+            raise ValueError("this batch does not fit the buffer's layout")
         tok_seq, tok_pos = [], []
         for b, (_, past, n, _) in enumerate(seqs):
             tok_seq += [b] * n
@@ -114,17 +133,21 @@ class BatchMeta:
         flat = tok_seq + tok_pos + self.start + [s[1] for s in seqs] + [s[0] for s in seqs]
         for *_, pg in seqs:
             flat += list(pg) + [0] * (self.max_pages - len(pg))
-        buf = torch.tensor(flat, dtype=torch.int32)
-        if device.type == "cuda":
-            buf = buf.pin_memory().to(device, non_blocking=True)
-        self.buf = buf
-        T, B = self.T, self.B
-        o = [0, T, 2 * T, 2 * T + B + 1, 2 * T + 2 * B + 1, 2 * T + 3 * B + 1]
-        self.tok_seq, self.tok_pos = buf[o[0]:o[1]], buf[o[1]:o[2]]
-        self.seq_start, self.seq_past, self.seq_slot = buf[o[2]:o[3]], buf[o[3]:o[4]], buf[o[4]:o[5]]
-        self.pages = buf[o[5]:].view(B, self.max_pages)
+        self._host.copy_(torch.tensor(flat, dtype=torch.int32))
+        if self.buf is not self._host:
+            self.buf.copy_(self._host, non_blocking=True)
         self._c = None
         self._split = {}
+        self._rot = {}
+
+    def cossin(self, inv_freq: torch.Tensor) -> torch.Tensor:
+        """[T, rot / 2, 2] float32: cos and sin of position * frequency for every row, made once per step and set of
+        frequencies with the library's full-precision functions (the angle itself is the float32 product)."""
+        key = inv_freq.data_ptr()
+        if key not in self._rot:
+            ang = self.tok_pos.to(inv_freq.device).float()[:, None] * inv_freq[None]
+            self._rot[key] = torch.stack([ang.cos(), ang.sin()], -1).contiguous()
+        return self._rot[key]
 
     def attn_split(self, min_rows: int):
         """Portions of at least ``min_rows`` rows as 64-row tiles [(sequence, first row)] for the matrix-core attention
@@ -137,8 +160,8 @@ class BatchMeta:
                 else:
                     rows += range(self.start[b], self.start[b] + n)
             buf = torch.tensor(tiles + rows + [0], dtype=torch.int32)
-            if self.buf.device.type == "cuda":
-                buf = buf.pin_memory().to(self.buf.device, non_blocking=True)
+            if self.device.type == "cuda":
+                buf = buf.pin_memory().to(self.device, non_blocking=True)
             self._split[min_rows] = (buf[:len(tiles)], len(tiles) // 2, buf[len(tiles):len(tiles) + len(rows)], len(rows))
         return self._split[min_rows]
 
@@ -225,7 +248,7 @@ class HipOps:
         if rot:
             if inv_freq.numel() != rot // 2:
                 raise ValueError("one frequency per rotated pair")
-            a.rot, a.inv_freq = rot, inv_freq.data_ptr()
+            a.rot, a.cossin = rot, meta.cossin(inv_freq).data_ptr()
         if out_dense is not None:
             if out_dense.shape != (meta.T, ngroups * gsize):
                 raise ValueError("dense output shape")

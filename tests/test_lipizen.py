@@ -452,3 +452,29 @@ def test_matrix_core_attention_against_the_plain_statement(H, G, d, e, window, k
     got = torch.cat(got).double().cpu().view(T, H, e)
     # the output is rounded to bfloat16 (2^-9 relative); the 32-bit softmax weights add nothing visible to that
     assert float((got - want).abs().max()) < 0.02 * float(want.abs().max()), float((got - want).abs().max())
+
+
+@pytest.mark.gpu
+def test_recorded_decode_steps_replay_like_eager_ones():
+    """Steps with one token per sequence are recorded into a hipGraph on their second occurrence and replayed from
+    then on.  Every replay is checked against the plain statement, with eager steps (prompt portions, another batch
+    size) between the replays, and against an engine that never records."""
+    cfg = full_model()
+    sd = O.random_weights(cfg, seed=101)
+    W = O.as_f64(sd)
+    prompts = {k: tokens(n, cfg["vocab"], 110 + i) for i, (k, n) in enumerate({"a": 90, "b": 40, "c": 75}.items())}
+    want = {k: O.forward(cfg, W, p) for k, p in prompts.items()}
+    schedule = [[("a", 60), ("b", 3)], [("a", 1), ("b", 1)], [("a", 1), ("b", 1)], [("a", 1), ("b", 1)], [("c", 20)],
+                [("a", 1), ("b", 1)], [("a", 1), ("b", 1), ("c", 1)], [("a", 1), ("b", 1), ("c", 1)], [("c", 30)],
+                [("a", 1), ("b", 1), ("c", 1)], [("a", 1), ("b", 1)], [("a", 1), ("b", 1)], [("a", 5), ("b", 1), ("c", 1)]]
+    schedule += [[("a", 1), ("b", 1)] for _ in range(17)] + [[("c", 1)] for _ in range(22)] + [[("b", 10)]]
+    eng = engine_for(cfg, sd, torch.float32, "cuda")
+    assert eng.use_graph
+    got = run_schedule(eng, prompts, schedule, 512, slots=3)
+    assert eng.graph_replays >= 30
+    plain = engine_for(cfg, sd, torch.float32, "cuda")
+    plain.use_graph = False
+    ref = run_schedule(plain, prompts, schedule, 512, slots=3)
+    for k in prompts:
+        close(got[k], want[k])
+        close(got[k], ref[k], 1e-4)
