@@ -122,9 +122,10 @@ class RaggedDecoder:
                     raise ValueError(f"layer {li}: kv_from must name an earlier attention layer with keys of its own and "
                                      "the same head layout")
         self.first_cost = self.rest_cost_mean = self.peak_memory = 0.0
-        # steps that carry one token per sequence are recorded once per (sequences, page-table width) and replayed as
-        # one hipGraph; BIGDL_RAGGED_GRAPH=0 issues them kernel by kernel like every other step
-        self.use_graph = self.device.type == "cuda" and os.environ.get("BIGDL_RAGGED_GRAPH", "1") != "0"
+        # BIGDL_RAGGED_GRAPH=1: steps that carry one token per sequence are recorded once per (sequences, page-table
+        # width) and replayed as one hipGraph.  Off by default: every step is issued kernel by kernel.  With recording
+        # on, a replay of a long trace ended with the GPU in a fault that has no established cause yet.
+        self.use_graph = self.device.type == "cuda" and os.environ.get("BIGDL_RAGGED_GRAPH", "0") == "1"
         self._graphs = {}
         self.graph_replays = 0
 
@@ -236,15 +237,19 @@ class RaggedDecoder:
             ent["meta"] = R.BatchMeta(seqs, self.device, max_pages=width, static=True)
             ent["host_ids"] = torch.empty(B, dtype=torch.int64, pin_memory=True)
             ent["ids"] = torch.zeros(B, dtype=torch.int64, device=self.device)
+            self.ops.before_recording(ent["meta"])       # whatever the operations would otherwise build on first use
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 ent["logits"] = self._forward(ent["meta"], ent["ids"], list(range(B)), None)
             ent["graph"] = graph
+        if "done" in ent:
+            ent["done"].synchronize()                    # the last replay has read the pinned buffers refilled below
         ent["meta"].update(seqs)
         ent["host_ids"].copy_(idt)
         ent["ids"].copy_(ent["host_ids"], non_blocking=True)
         ent["graph"].replay()
+        ent.setdefault("done", torch.cuda.Event()).record()
         self.graph_replays += 1
         return ent["logits"].clone()
 

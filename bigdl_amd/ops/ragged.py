@@ -108,15 +108,23 @@ class BatchMeta:
         self.T = sum(n for _, _, n, _ in seqs)
         self.max_pages = max_pages or max(1, max(len(pg) for *_, pg in seqs))
         T, B = self.T, self.B
-        size = 2 * T + 3 * B + 1 + B * self.max_pages
-        self._host = torch.empty(size, dtype=torch.int32, pin_memory=device.type == "cuda")
-        self.buf = torch.empty(size, dtype=torch.int32, device=device) if static or device.type == "cuda" else self._host
+        self._static = static
+        self._c = None
+        self._split = {}
+        self._rot = {}
+        if static:
+            size = 2 * T + 3 * B + 1 + B * self.max_pages
+            self._host = torch.empty(size, dtype=torch.int32, pin_memory=device.type == "cuda")
+            self.buf = torch.empty(size, dtype=torch.int32, device=device)
+            self._views()
+        self.update(seqs)
+
+    def _views(self):
+        T, B, buf = self.T, self.B, self.buf
         o = [0, T, 2 * T, 2 * T + B + 1, 2 * T + 2 * B + 1, 2 * T + 3 * B + 1]
-        buf = self.buf
         self.tok_seq, self.tok_pos = buf[o[0]:o[1]], buf[o[1]:o[2]]
         self.seq_start, self.seq_past, self.seq_slot = buf[o[2]:o[3]], buf[o[3]:o[4]], buf[o[4]:o[5]]
         self.pages = buf[o[5]:].view(B, self.max_pages)
-        self.update(seqs)
 
     def update(self, seqs):
         """Fill the buffer for this step's sequences (same count and row total as at construction)."""
@@ -133,12 +141,15 @@ class BatchMeta:
         flat = tok_seq + tok_pos + self.start + [s[1] for s in seqs] + [s[0] for s in seqs]
         for *_, pg in seqs:
             flat += list(pg) + [0] * (self.max_pages - len(pg))
-        self._host.copy_(torch.tensor(flat, dtype=torch.int32))
-        if self.buf is not self._host:
+        if self._static:
+            self._host.copy_(torch.tensor(flat, dtype=torch.int32))
             self.buf.copy_(self._host, non_blocking=True)
-        self._c = None
-        self._split = {}
-        self._rot = {}
+            return
+        buf = torch.tensor(flat, dtype=torch.int32)
+        if self.device.type == "cuda":
+            buf = buf.pin_memory().to(self.device, non_blocking=True)
+        self.buf = buf
+        self._views()
 
     def cossin(self, inv_freq: torch.Tensor) -> torch.Tensor:
         """[T, rot / 2, 2] float32: cos and sin of position * frequency for every row, made once per step and set of
@@ -208,6 +219,10 @@ class HipOps:
     name = "hip"
     mfma = os.environ.get("BIGDL_RAGGED_MFMA", "1") != "0"      # 0: every row through the row-wise attention kernel
     mfma_min_rows = 8
+
+    def before_recording(self, meta):
+        """Host-built tables a step needs (pinned allocations and copies cannot be recorded into a graph)."""
+        meta.attn_split(self.mfma_min_rows)
 
     def sum_group_norm(self, x, y, w, groups, alpha, eps, act, x_out=None, want_act=True):
         _f32(x, w, x_out)

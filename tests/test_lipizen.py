@@ -455,6 +455,9 @@ def test_matrix_core_attention_against_the_plain_statement(H, G, d, e, window, k
 
 
 @pytest.mark.gpu
+@pytest.mark.skip(reason="recording of decode steps is off by default (BIGDL_RAGGED_GRAPH=1): this test passed on the GPU, "
+                         "but a long trace replayed with recording on left the GPU in a fault whose cause is not "
+                         "established; the path stays off the GPU until it is")
 def test_recorded_decode_steps_replay_like_eager_ones():
     """Steps with one token per sequence are recorded into a hipGraph on their second occurrence and replayed from
     then on.  Every replay is checked against the plain statement, with eager steps (prompt portions, another batch
@@ -462,14 +465,14 @@ def test_recorded_decode_steps_replay_like_eager_ones():
     cfg = full_model()
     sd = O.random_weights(cfg, seed=101)
     W = O.as_f64(sd)
-    prompts = {k: tokens(n, cfg["vocab"], 110 + i) for i, (k, n) in enumerate({"a": 90, "b": 40, "c": 75}.items())}
+    prompts = {k: tokens(n, cfg["vocab"], 110 + i) for i, (k, n) in enumerate({"a": 91, "b": 40, "c": 76}.items())}
     want = {k: O.forward(cfg, W, p) for k, p in prompts.items()}
     schedule = [[("a", 60), ("b", 3)], [("a", 1), ("b", 1)], [("a", 1), ("b", 1)], [("a", 1), ("b", 1)], [("c", 20)],
                 [("a", 1), ("b", 1)], [("a", 1), ("b", 1), ("c", 1)], [("a", 1), ("b", 1), ("c", 1)], [("c", 30)],
                 [("a", 1), ("b", 1), ("c", 1)], [("a", 1), ("b", 1)], [("a", 1), ("b", 1)], [("a", 5), ("b", 1), ("c", 1)]]
     schedule += [[("a", 1), ("b", 1)] for _ in range(17)] + [[("c", 1)] for _ in range(22)] + [[("b", 10)]]
     eng = engine_for(cfg, sd, torch.float32, "cuda")
-    assert eng.use_graph
+    eng.use_graph = True
     got = run_schedule(eng, prompts, schedule, 512, slots=3)
     assert eng.graph_replays >= 30
     plain = engine_for(cfg, sd, torch.float32, "cuda")
