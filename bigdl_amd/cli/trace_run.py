@@ -53,6 +53,8 @@ def main(argv=None) -> int:
         for e in msg.get("entries", []):
             if e["id"] not in slot_of:
                 slot_of[e["id"]] = pool.admit()
+            if not e.get("tokens"):
+                continue                                   # admitted, nothing to run for it in this step
             entries.append((slot_of[e["id"]], e["tokens"]))
             want.append(list(e.get("want") or []))
         if entries:
