@@ -75,14 +75,19 @@ def close(a, b, tol=F32_TOL):
     [O.attention_layer(ff=0)], [O.hgrn2_layer()], [O.attention_layer()], [O.hgrn2_layer(ff=40)],
     [O.attention_layer(heads=3, kv_heads=3, dim=24, vdim=80, conv=0, size=None, rot_dims=24, factor=1.0, diff=0.8)],
     [O.attention_layer(heads=6, kv_heads=1, dim=20, vdim=12, conv=2, size=200, keep_first=0, rot_dims=0)],
-], ids=["attention", "hgrn2", "attention+ff", "hgrn2+ff", "full-mask-wide-values", "one-kv-head-no-rotation"])
+    [O.attention_layer(heads=2, kv_heads=1, dim=18, vdim=15, conv=3, size=10, keep_first=1, rot_dims=6)],
+    [O.attention_layer(heads=8, kv_heads=1, dim=32, vdim=272, conv=1, size=33, keep_first=70, rot_dims=32, ff=0)],
+    [O.attention_layer(heads=8, kv_heads=1, dim=32, vdim=64, conv=2, size=70, keep_first=2, rot_dims=16, ff=0),
+     O.attention_layer(heads=6, kv_heads=3, dim=64, vdim=192, conv=0, size=40, keep_first=0, rot_dims=0, ff=0)],
+], ids=["attention", "hgrn2", "attention+ff", "hgrn2+ff", "full-mask-wide-values", "one-kv-head-no-rotation",
+        "odd-sizes", "eight-heads-per-kv-head-very-wide-values", "shared-reads-of-8-and-2-heads"])
 def test_each_layer_kind_alone(device, layers):
     cfg = O.make_config(layers, groups=1 if len(layers[0]["mixer"]) < 4 else 2)
     sd = O.random_weights(cfg, seed=1)
-    toks = tokens(45, cfg["vocab"], 2)
+    toks = tokens(85, cfg["vocab"], 2)
     want = O.forward(cfg, O.as_f64(sd), toks)
     eng = engine_for(cfg, sd, torch.float32, device)
-    got = run_schedule(eng, {"a": toks}, [[("a", len(toks))]], 64)["a"]
+    got = run_schedule(eng, {"a": toks}, [[("a", 45)], [("a", 38)], [("a", 1)], [("a", 1)]], 128)["a"]
     close(got, want)
 
 
@@ -153,8 +158,13 @@ def test_long_decoding_past_windows_and_pages(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-def test_bfloat16_stays_near_the_exact_result(device):
+@pytest.mark.parametrize("odd", [False, True])
+def test_bfloat16_stays_near_the_exact_result(device, odd):
     cfg = full_model()
+    if odd:          # sizes that take none of the vector or matrix-core paths
+        cfg = O.make_config([O.attention_layer(heads=2, kv_heads=1, dim=20, vdim=30, rot_dims=10),
+                             O.hgrn2_layer(heads=1, dim=36, vdim=20), O.attention_layer(heads=2, kv_heads=1, dim=20, vdim=30,
+                                                                                        rot_dims=10, kv_from=0, conv=0)])
     sd = O.random_weights(cfg, seed=13)
     toks = tokens(100, cfg["vocab"], 14)
     want = O.forward(cfg, O.as_f64(sd), toks)
