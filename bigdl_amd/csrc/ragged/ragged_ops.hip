@@ -358,6 +358,52 @@ extern "C" int ragged_hgrn2_scan(const float* qf, const float* ff, const void* P
   return RAGGED_LAUNCH_OK();
 }
 
+// Long portions: the scan is cut into chunks that run side by side.  Every chunk is scanned from a zero state (its
+// local end state L_c), the product D_c of its gates is taken per row, the true state at every chunk's start follows
+// from S_(c+1) = diag(D_c) S_c + L_c, and the chunks are scanned again from those states for the outputs.  Nothing is
+// divided, so small gate products only fade a contribution out.  The scans are hgrn2_scan_kernel over a batch whose
+// "sequences" are the chunks and whose "slots" are rows of a scratch state array.
+__global__ __launch_bounds__(256) void hgrn2_chunk_decay_kernel(const float* __restrict__ ff, const int* __restrict__ cstart,
+                                                                float* __restrict__ decay, int HD) {
+  const int c = blockIdx.x, ch = blockIdx.y * 256 + threadIdx.x;
+  if (ch >= HD) return;
+  float p = 1.f;
+  for (int t = cstart[c]; t < cstart[c + 1]; ++t) p *= ff[(int64_t)t * HD + ch];
+  decay[(int64_t)c * HD + ch] = p;
+}
+
+// one thread per state element of a real sequence; cfirst[b] .. cfirst[b + 1] - 1 are its chunks
+__global__ __launch_bounds__(256) void hgrn2_chunk_combine_kernel(const float* __restrict__ state, const float* __restrict__ local,
+                                                                  const float* __restrict__ decay, float* __restrict__ begin,
+                                                                  const int* __restrict__ cfirst, const int* __restrict__ seq_past,
+                                                                  const int* __restrict__ seq_slot, int H, int d, int vd) {
+  const int b = blockIdx.y;
+  const int64_t E = (int64_t)H * d * vd, e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= E) return;
+  const int hrow = (int)(e / vd);                          // h * d + row
+  float S = seq_past[b] > 0 ? state[(int64_t)seq_slot[b] * E + e] : 0.f;
+  for (int c = cfirst[b]; c < cfirst[b + 1]; ++c) {
+    begin[(int64_t)c * E + e] = S;
+    S = decay[(int64_t)c * H * d + hrow] * S + local[(int64_t)c * E + e];
+  }
+}
+
+extern "C" int ragged_hgrn2_chunk_decay(const float* ff, const int* cstart, float* decay, int n_chunks, int HD, hipStream_t st) {
+  if (n_chunks <= 0 || HD <= 0) return -1;
+  hipLaunchKernelGGL(hgrn2_chunk_decay_kernel, dim3(n_chunks, (HD + 255) / 256), dim3(256), 0, st, ff, cstart, decay, HD);
+  return RAGGED_LAUNCH_OK();
+}
+
+extern "C" int ragged_hgrn2_chunk_combine(const float* state, const float* local, const float* decay, float* begin,
+                                          const int* cfirst, const int* seq_past, const int* seq_slot, int B, int H, int d, int vd,
+                                          hipStream_t st) {
+  if (B <= 0 || H <= 0 || d <= 0 || vd <= 0) return -1;
+  const int64_t E = (int64_t)H * d * vd;
+  hipLaunchKernelGGL(hgrn2_chunk_combine_kernel, dim3((unsigned)((E + 255) / 256), B), dim3(256), 0, st, state, local, decay, begin,
+                     cfirst, seq_past, seq_slot, H, d, vd);
+  return RAGGED_LAUNCH_OK();
+}
+
 // RMS norm over rows of `n` floats with a weight (or none), output of type T.  One wavefront per row.
 template <typename T>
 __global__ __launch_bounds__(256) void row_norm_kernel(const float* __restrict__ x, const float* __restrict__ w, T* __restrict__ out,

@@ -88,6 +88,8 @@ def lib():
         L.ragged_clamped_glu.argtypes = [vp, vp, i64, ci, cf, cf, ci, vp]
         L.ragged_hgrn2_gates.argtypes = [vp, i64, ci, ci, vp, vp, vp, vp, i64, ci, ci, vp]
         L.ragged_hgrn2_scan.argtypes = [vp, vp, vp, i64, ci, vp, vp, ci, ci, ci, _Batch, ci, vp]
+        L.ragged_hgrn2_chunk_decay.argtypes = [vp, vp, vp, ci, ci, vp]
+        L.ragged_hgrn2_chunk_combine.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, vp]
         L.ragged_row_norm.argtypes = [vp, vp, vp, i64, ci, cf, ci, vp]
         L.ragged_paged_attn.argtypes = [_AttnArgs, _Batch, ci, ci, vp]
         L.ragged_paged_attn_mfma.argtypes = [_AttnArgs, _Batch, ci, vp]
@@ -112,6 +114,7 @@ class BatchMeta:
         self._c = None
         self._split = {}
         self._rot = {}
+        self._chunks = {}
         if static:
             size = 2 * T + 3 * B + 1 + B * self.max_pages
             self._host = torch.empty(size, dtype=torch.int32, pin_memory=device.type == "cuda")
@@ -150,6 +153,26 @@ class BatchMeta:
             buf = buf.pin_memory().to(self.device, non_blocking=True)
         self.buf = buf
         self._views()
+
+    def chunks(self, length: int):
+        """Every sequence's rows cut into chunks of ``length``: (number of chunks, device int32 arrays
+        chunk_start[NC + 1] (token rows), zeros[NC], ones[NC], chunk_id[NC], first_chunk_of_sequence[B + 1]) and the
+        host list of each sequence's last chunk."""
+        if length not in self._chunks:
+            cstart, cfirst, last = [0], [0], []
+            for _, _, n, _ in self.seqs:
+                for c0 in range(0, n, length):
+                    cstart.append(cstart[-1] + min(length, n - c0))
+                cfirst.append(len(cstart) - 1)
+                last.append(len(cstart) - 2)
+            nc = len(cstart) - 1
+            flat = cstart + [0] * nc + [1] * nc + list(range(nc)) + cfirst
+            buf = torch.tensor(flat, dtype=torch.int32)
+            if self.device.type == "cuda":
+                buf = buf.pin_memory().to(self.device, non_blocking=True)
+            o = [0, nc + 1, 2 * nc + 1, 3 * nc + 1, 4 * nc + 1]
+            self._chunks[length] = (nc, buf[o[0]:o[1]], buf[o[1]:o[2]], buf[o[2]:o[3]], buf[o[3]:o[4]], buf[o[4]:], last)
+        return self._chunks[length]
 
     def cossin(self, inv_freq: torch.Tensor) -> torch.Tensor:
         """[T, rot / 2, 2] float32: cos and sin of position * frequency for every row, made once per step and set of
@@ -219,6 +242,7 @@ class HipOps:
     name = "hip"
     mfma = os.environ.get("BIGDL_RAGGED_MFMA", "1") != "0"      # 0: every row through the row-wise attention kernel
     mfma_min_rows = 8
+    scan_chunk = 256          # portions of at least twice this many tokens run their recurrence in chunks
 
     def before_recording(self, meta):
         """Host-built tables a step needs (pinned allocations and copies cannot be recorded into a graph)."""
@@ -313,8 +337,30 @@ class HipOps:
                 or state.shape[1:] != (H, d, vd) or max(s[0] for s in meta.seqs) >= state.shape[0]:
             raise ValueError("recurrent state / gates do not fit")
         out = torch.empty(meta.T, H * vd, dtype=torch.float32, device=P.device)
-        _ok(lib().ragged_hgrn2_scan(qf.data_ptr(), ff.data_ptr(), P.data_ptr(), P.stride(0), v0, state.data_ptr(),
-                                    out.data_ptr(), H, d, vd, meta.c(), _DT[P.dtype], _stream()), "hgrn2_scan")
+        L, dt, st = lib(), _DT[P.dtype], _stream()
+        longest = max(n for _, _, n, _ in meta.seqs)
+        if longest < 2 * self.scan_chunk:
+            _ok(L.ragged_hgrn2_scan(qf.data_ptr(), ff.data_ptr(), P.data_ptr(), P.stride(0), v0, state.data_ptr(),
+                                    out.data_ptr(), H, d, vd, meta.c(), dt, st), "hgrn2_scan")
+            return out
+        # long portions: chunks scanned side by side from zero, chunk-start states chained, chunks scanned again from them
+        nc, cstart, zeros, ones, cid, cfirst, last = meta.chunks(self.scan_chunk)
+        local = torch.empty(nc, H, d, vd, dtype=torch.float32, device=P.device)
+        begin = torch.empty_like(local)
+        decay = torch.empty(nc, H * d, dtype=torch.float32, device=P.device)
+
+        def chunk_batch(past):
+            return _Batch(None, None, cstart.data_ptr(), past.data_ptr(), cid.data_ptr(), None, meta.T, nc, 0)
+        _ok(L.ragged_hgrn2_scan(qf.data_ptr(), ff.data_ptr(), P.data_ptr(), P.stride(0), v0, local.data_ptr(), out.data_ptr(),
+                                H, d, vd, chunk_batch(zeros), dt, st), "hgrn2_scan (chunks from zero)")
+        _ok(L.ragged_hgrn2_chunk_decay(ff.data_ptr(), cstart.data_ptr(), decay.data_ptr(), nc, H * d, st), "hgrn2_chunk_decay")
+        _ok(L.ragged_hgrn2_chunk_combine(state.data_ptr(), local.data_ptr(), decay.data_ptr(), begin.data_ptr(), cfirst.data_ptr(),
+                                         meta.seq_past.data_ptr(), meta.seq_slot.data_ptr(), meta.B, H, d, vd, st),
+            "hgrn2_chunk_combine")
+        _ok(L.ragged_hgrn2_scan(qf.data_ptr(), ff.data_ptr(), P.data_ptr(), P.stride(0), v0, begin.data_ptr(), out.data_ptr(),
+                                H, d, vd, chunk_batch(ones), dt, st), "hgrn2_scan (chunks from their start states)")
+        slots = torch.tensor([s[0] for s in meta.seqs], dtype=torch.int64, device=P.device)
+        state[slots] = begin[torch.tensor(last, dtype=torch.int64, device=P.device)]     # every sequence's end state
         return out
 
     def row_norm(self, x, w, eps, act):

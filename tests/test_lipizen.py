@@ -146,6 +146,20 @@ def test_unequal_requests_in_one_batch_and_reuse_of_pages_and_slots(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+def test_long_and_short_portions_side_by_side_through_the_recurrence(device):
+    """a portion long enough for the chunked scan next to a short one and a single token, then the long one goes on"""
+    cfg = O.make_config([O.hgrn2_layer(heads=2, dim=24, vdim=20, ff=32), O.hgrn2_layer(heads=1, dim=70, vdim=33)])
+    sd = O.random_weights(cfg, seed=17)
+    W = O.as_f64(sd)
+    prompts = {"a": tokens(1400, cfg["vocab"], 18), "b": tokens(41, cfg["vocab"], 19), "c": tokens(3, cfg["vocab"], 20)}
+    want = {k: O.forward(cfg, W, p) for k, p in prompts.items()}
+    eng = engine_for(cfg, sd, torch.float32, device)
+    got = run_schedule(eng, prompts, [[("c", 2), ("a", 700), ("b", 40)], [("a", 1), ("b", 1), ("c", 1)], [("a", 699)]], 1600)
+    for k in prompts:
+        close(got[k], want[k])
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_long_decoding_past_windows_and_pages(device):
     cfg = O.make_config([O.attention_layer(size=16, keep_first=3), O.hgrn2_layer(),
                          O.attention_layer(size=70, keep_first=1, kv_from=0)])
@@ -274,13 +288,15 @@ def test_short_convolution_norm_rotation_and_state(device, taps, portions):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("heads,dim,vdim", [(2, 16, 16), (1, 40, 24), (3, 80, 70), (1, 8, 130)])
-def test_hgrn2_recurrence_and_its_state(device, heads, dim, vdim):
+@pytest.mark.parametrize("heads,dim,vdim,portions", [(2, 16, 16, (1, 2, 64, 1, 22)), (1, 40, 24, (1, 2, 64, 1, 22)),
+                                                     (3, 80, 70, (1, 2, 64, 1, 22)), (1, 8, 130, (1, 2, 64, 1, 22)),
+                                                     (2, 48, 40, (530, 3, 700))])
+def test_hgrn2_recurrence_and_its_state(device, heads, dim, vdim, portions):
     g = torch.Generator().manual_seed(41)
     cfg = O.make_config([O.hgrn2_layer(heads=heads, dim=dim, vdim=vdim)], width=32)
     sd = O.random_weights(cfg, seed=42)
     W = O.as_f64(sd)
-    T = 90
+    T = sum(portions)                      # (portions of 512 tokens and more run in chunks on the GPU)
     h = torch.randn(T, 32, generator=g, dtype=O.F64)
     m = cfg["layers"][0]["mixer"]
     # the oracle's mixer up to (not including) the output norm and projection
@@ -295,14 +311,14 @@ def test_hgrn2_recurrence_and_its_state(device, heads, dim, vdim):
         S = f[t][:, :, None] * S + (1 - f[t])[:, :, None] * v[t].view(heads, 1, vdim)
         want[t] = torch.einsum("hde,hd->he", S, q[t].view(heads, dim))
     ops = R.ops_for(device)
-    pool = PagedStatePool({0: [("matrix", heads, dim, vdim)]}, 128, 2, torch.float32, device)
+    pool = PagedStatePool({0: [("matrix", heads, dim, vdim)]}, T + 64, 2, torch.float32, device)
     pool.admit()
     slot = pool.admit()
     pool.matrix[0].fill_(3.0)                                # left by an earlier sequence: must not leak in
     P = torch.cat([h @ W["l0.mix.q"].T, fpre, v], 1).float().to(device).contiguous()
     hd = heads * dim
     out, at = [], 0
-    for n in (1, 2, 64, 1, 22):
+    for n in portions:
         meta = _meta_for(pool, slot, n, device)
         Pn = P[at:at + n].contiguous()
         qf, ff = ops.hgrn2_gates(Pn, 0, hd, W["l0.mix.f.b"].float().to(device), low.float().to(device), hd)
