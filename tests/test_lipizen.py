@@ -79,8 +79,11 @@ def close(a, b, tol=F32_TOL):
     [O.attention_layer(heads=8, kv_heads=1, dim=32, vdim=272, conv=1, size=33, keep_first=70, rot_dims=32, ff=0)],
     [O.attention_layer(heads=8, kv_heads=1, dim=32, vdim=64, conv=2, size=70, keep_first=2, rot_dims=16, ff=0),
      O.attention_layer(heads=6, kv_heads=3, dim=64, vdim=192, conv=0, size=40, keep_first=0, rot_dims=0, ff=0)],
+    [O.attention_layer(heads=4, kv_heads=2, dim=12, vdim=20, conv=3, size=30, keep_first=2, rot_dims=12, ff=0),
+     O.attention_layer(heads=8, kv_heads=2, dim=24, vdim=200, conv=3, size=30, keep_first=2, rot_dims=8, ff=0)],
 ], ids=["attention", "hgrn2", "attention+ff", "hgrn2+ff", "full-mask-wide-values", "one-kv-head-no-rotation",
-        "odd-sizes", "eight-heads-per-kv-head-very-wide-values", "shared-reads-of-8-and-2-heads"])
+        "odd-sizes", "eight-heads-per-kv-head-very-wide-values", "shared-reads-of-8-and-2-heads",
+        "key-rows-that-do-not-divide-a-wavefront"])
 def test_each_layer_kind_alone(device, layers):
     cfg = O.make_config(layers, groups=1 if len(layers[0]["mixer"]) < 4 else 2)
     sd = O.random_weights(cfg, seed=1)
@@ -437,7 +440,7 @@ def test_trace_runner_replays_steps(tmp_path):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("H,G,d,e,window,keep", [(4, 2, 64, 128, 100, 5), (2, 2, 48, 96, 70, 0), (3, 1, 16, 32, 0, 0),
+@pytest.mark.parametrize("H,G,d,e,window,keep", [(4, 2, 64, 128, 100, 5), (2, 2, 48, 96, 70, 0), (4, 1, 48, 96, 70, 3), (3, 1, 16, 32, 0, 0),
                                                  (2, 1, 128, 64, 300, 70), (2, 2, 40, 16, 64, 64)])
 def test_matrix_core_attention_against_the_plain_statement(H, G, d, e, window, keep):
     """bfloat16 prompt portions take the MFMA kernel, single tokens the row-wise one: both against float64 attention
