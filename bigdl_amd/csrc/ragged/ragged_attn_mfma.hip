@@ -6,10 +6,12 @@
 //    column) and 4 keys of each 16-key block: running maximum, normaliser and rescale factor are per-lane scalars
 //    (two cross-lane steps join the 4 lanes of a query), and the exponentials are already laid out as the B operand of
 //    the second product O^T += V^T P^T, with the keys of a 32-key chunk in the order (4 g + j, 16 + 4 g + j).
-//  * K fragments come straight from the page (16 bytes per lane); the value tile is transposed into LDS once per page
-//    by the whole workgroup and read back as A fragments (two 8-byte reads per fragment).
-//  * softmax weights stay 32-bit quantities: each is split into two bfloat16 terms (p = hi + lo) that go through the
-//    matrix core one after the other, so the second product loses nothing beyond the values' own 16 bits.
+//  * K fragments come straight from the page (16 bytes per lane), requested one page ahead; the value tile is transposed into LDS once per page by the whole
+//    workgroup (a lane per key, so the 2-byte stores of a wavefront fall into consecutive addresses) from registers
+//    that were loaded during the previous page's arithmetic, and read back as A fragments (two 8-byte reads each).
+//  * softmax weights stay 32-bit quantities up to the matrix core: each goes through it as two bfloat16 terms, the upper
+//    16 bits of p and the upper 16 bits of the exact remainder (2^-16 relative), so the second product loses nothing
+//    beyond the values' own 16 bits.
 //  * both maps of a differential head share the K page walk and the value tile.
 #include "ragged_attn.h"
 
@@ -32,7 +34,7 @@ union Frag {
 
 __device__ __forceinline__ uint16_t bf_bits(float f) { return from_f<bf16>(f).b; }
 
-template <int MAPS>
+template <int MAPS, int DK>
 __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch bt) {
   __shared__ __attribute__((aligned(16))) uint16_t vt[MF_NEB * 16 * MF_LDV];      // V^T [vd][PAGE (+ pad)]
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -42,7 +44,7 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
   const int start = bt.seq_start[b], n = bt.seq_start[b + 1] - start, past = bt.seq_past[b];
   const int gk = h / (a.H / a.G);
   const int qd = MAPS * a.d;
-  const int dk = (a.d + 31) / 32, neb = a.vd / 16;
+  const int neb = a.vd / 16;
   const int nrows = n - row0 < 64 ? n - row0 : 64;          // rows of this tile
   const int myrow = row0 + 16 * wave + lq;                  // this lane's query inside the portion
   const bool rowok = 16 * wave + lq < nrows;
@@ -50,15 +52,15 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
   const int64_t t = start + (rowok ? myrow : row0);
 
   // queries as B fragments: lane = query lq, channels 32 ks + 8 g4 .. + 7
-  Frag qf[MAPS][MF_DK];
+  Frag qf[MAPS][DK];
 #pragma unroll
   for (int mp = 0; mp < MAPS; ++mp)
 #pragma unroll
-    for (int ks = 0; ks < MF_DK; ++ks) {
+    for (int ks = 0; ks < DK; ++ks) {
       const int ch = 32 * ks + 8 * g4;
 #pragma unroll
       for (int e = 0; e < 4; ++e) qf[mp][ks].u[e] = 0;
-      if (ks < dk && ch < a.d && rowok) {
+      if (ch < a.d && rowok) {
         const float* qp = a.q + ((t * a.H + h) * MAPS + mp) * a.d + ch;
 #pragma unroll
         for (int e = 0; e < 8; ++e) qf[mp][ks].h[e] = bf_bits(qp[e]);
@@ -92,33 +94,24 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
     for (int eb = 0; eb < MF_NEB; ++eb) O[mp][eb] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int o = 0; o < npg; ++o) {
-    const int pg = o < kept_pages ? o : pl + (o - kept_pages);
-    const int page = pages[pg];
-    const int k0 = pg * PAGE;
-    // ---- value tile -> LDS, transposed
-    __syncthreads();                                         // the previous page's fragments have been read
-    {
-      const bf16* vsrc = V + (((int64_t)page * a.G + gk) * PAGE) * a.vd;
-      const int total = PAGE * a.vd;
-      for (int idx = threadIdx.x * 8; idx < total; idx += 256 * 8) {
-        const int key = idx / a.vd, e0 = idx % a.vd;
-        Frag f;
-        f.q = *reinterpret_cast<const uint4*>(vsrc + idx);
+  // value tile of a page: lane = key, wavefront w takes channel groups w, w + 4, ... (8 channels = 16 bytes each)
+  Frag vreg[4];
+  auto page_of = [&](int o) { return pages[o < kept_pages ? o : pl + (o - kept_pages)]; };
+  auto load_values = [&](int page) {
+    const bf16* vsrc = V + (((int64_t)page * a.G + gk) * PAGE + lane) * a.vd;
 #pragma unroll
-        for (int u = 0; u < 8; ++u) vt[(e0 + u) * MF_LDV + key] = f.h[u];
-      }
+    for (int it = 0; it < 4; ++it) {
+      const int e0 = 8 * (4 * it + wave);
+      if (e0 < a.vd) vreg[it].q = *reinterpret_cast<const uint4*>(vsrc + e0);
     }
-    __syncthreads();
-    const bool wave_sees = wave_has_rows && k0 <= w_last && (k0 + PAGE - 1 >= w_lo || k0 < keep);
-    if (!wave_sees) continue;
-
-    // ---- S^T = K Q^T for the 4 key blocks of the page
-    f32x4 S[MAPS][4];
-#pragma unroll
-    for (int mp = 0; mp < MAPS; ++mp)
-#pragma unroll
-      for (int kb = 0; kb < 4; ++kb) S[mp][kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  };
+  // K fragments of a page: 16 bytes per lane and (key block, map, 32-channel step), requested one page ahead
+  Frag kf[4][MAPS][DK], kfn[4][MAPS][DK];
+  auto sees = [&](int o) {
+    const int k0 = (o < kept_pages ? o : pl + (o - kept_pages)) * PAGE;
+    return wave_has_rows && k0 <= w_last && (k0 + PAGE - 1 >= w_lo || k0 < keep);
+  };
+  auto load_keys = [&](int page) {
     const bf16* kpage = K + (((int64_t)page * a.G + gk) * PAGE) * qd;
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
@@ -126,30 +119,81 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
 #pragma unroll
       for (int mp = 0; mp < MAPS; ++mp)
 #pragma unroll
-        for (int ks = 0; ks < MF_DK; ++ks) {
+        for (int ks = 0; ks < DK; ++ks) {
           const int ch = 32 * ks + 8 * g4;
-          if (ks < dk) {
-            Frag kf;
-            kf.q = ch < a.d ? *reinterpret_cast<const uint4*>(krow + mp * a.d + ch) : uint4{0, 0, 0, 0};
-            S[mp][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[mp][ks].v, S[mp][kb], 0, 0, 0);
-          }
+          kfn[kb][mp][ks].q = ch < a.d ? *reinterpret_cast<const uint4*>(krow + mp * a.d + ch) : uint4{0, 0, 0, 0};
         }
     }
+  };
+  if (npg > 0) {
+    load_values(page_of(0));
+    if (sees(0)) load_keys(page_of(0));
+  }
+
+  for (int o = 0; o < npg; ++o) {
+    const int pg = o < kept_pages ? o : pl + (o - kept_pages);
+    const int k0 = pg * PAGE;
+    const bool wave_sees = sees(o);
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int mp = 0; mp < MAPS; ++mp)
+#pragma unroll
+        for (int ks = 0; ks < DK; ++ks) kf[kb][mp][ks].q = kfn[kb][mp][ks].q;
+    // ---- value tile -> LDS, transposed
+    __syncthreads();                                         // the previous page's fragments have been read
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int e0 = 8 * (4 * it + wave);
+      if (e0 < a.vd) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) vt[(e0 + u) * MF_LDV + lane] = vreg[it].h[u];
+      }
+    }
+    __syncthreads();
+    if (o + 1 < npg) {                                       // in flight during this page's arithmetic
+      load_values(page_of(o + 1));
+      if (sees(o + 1)) load_keys(page_of(o + 1));
+    }
+    if (!wave_sees) continue;
+
+    // ---- S^T = K Q^T for the 4 key blocks of the page
+    f32x4 S[MAPS][4];
+#pragma unroll
+    for (int mp = 0; mp < MAPS; ++mp)
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        S[mp][kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < DK; ++ks)
+          S[mp][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kb][mp][ks].v, qf[mp][ks].v, S[mp][kb], 0, 0, 0);
+      }
     // ---- mask, online softmax (per-lane scalars of the lane's query), exponentials as two bfloat16 terms
     Frag phi[MAPS][2], plo[MAPS][2];
+    // a page whose 64 keys every row of this wavefront sees needs no mask arithmetic
+    const bool inner = k0 + PAGE - 1 <= w_first && (!win || k0 >= w_last - a.window + 1 || k0 + PAGE - 1 < keep);
 #pragma unroll
     for (int mp = 0; mp < MAPS; ++mp) {
       float mx = -1e30f;
-      bool vis[4][4];
+      if (inner) {
 #pragma unroll
-      for (int kb = 0; kb < 4; ++kb)
+        for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = k0 + 16 * kb + 4 * g4 + i;
-          vis[kb][i] = key <= qpos && (key >= my_lo || key < keep);
-          S[mp][kb][i] = vis[kb][i] ? S[mp][kb][i] * a.scale : -1e30f;
-          mx = fmaxf(mx, S[mp][kb][i]);
-        }
+          for (int i = 0; i < 4; ++i) {
+            S[mp][kb][i] *= a.scale;
+            mx = fmaxf(mx, S[mp][kb][i]);
+          }
+      } else {
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = k0 + 16 * kb + 4 * g4 + i;
+            const bool vis = key <= qpos && (key >= my_lo || key < keep);
+            S[mp][kb][i] = vis ? S[mp][kb][i] * a.scale : -1e30f;
+            mx = fmaxf(mx, S[mp][kb][i]);
+          }
+      }
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       const float mnew = fmaxf(m[mp], mx);
@@ -158,13 +202,16 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float p = vis[kb][i] ? __expf(S[mp][kb][i] - mnew) : 0.f;
-          sum += p;
-          const uint16_t hi = bf_bits(p);
-          const float rest = p - __uint_as_float((uint32_t)hi << 16);
-          phi[mp][kb >> 1].h[4 * (kb & 1) + i] = hi;
-          plo[mp][kb >> 1].h[4 * (kb & 1) + i] = bf_bits(rest);
+        for (int i = 0; i < 4; i += 2) {
+          // masked scores are -1e30: their exponential is 0 unless the row has seen no key yet (mnew = -1e30)
+          float p0 = S[mp][kb][i] > -1e29f ? __expf(S[mp][kb][i] - mnew) : 0.f;
+          float p1 = S[mp][kb][i + 1] > -1e29f ? __expf(S[mp][kb][i + 1] - mnew) : 0.f;
+          sum += p0 + p1;
+          // p = hi + lo with hi the upper 16 bits of p (exact remainder) and lo the upper 16 bits of the remainder
+          const uint32_t h0 = __float_as_uint(p0) & 0xffff0000u, h1 = __float_as_uint(p1) & 0xffff0000u;
+          const uint32_t l0 = __float_as_uint(p0 - __uint_as_float(h0)), l1 = __float_as_uint(p1 - __uint_as_float(h1));
+          phi[mp][kb >> 1].u[2 * (kb & 1) + (i >> 1)] = (h0 >> 16) | h1;
+          plo[mp][kb >> 1].u[2 * (kb & 1) + (i >> 1)] = (l0 >> 16) | (l1 & 0xffff0000u);
         }
       sum += __shfl_xor(sum, 16, 64);
       sum += __shfl_xor(sum, 32, 64);
@@ -228,11 +275,20 @@ extern "C" int ragged_paged_attn_mfma_ok(int d, int vd) {
   return d % 8 == 0 && d <= 32 * MF_DK && vd % 16 == 0 && vd <= 16 * MF_NEB;
 }
 
+template <int MAPS>
+static void launch_mfma(AttnArgs a, Batch bt, unsigned grid, hipStream_t st) {
+  const int dk = (a.d + 31) / 32;
+  if (dk == 1) hipLaunchKernelGGL((paged_attn_mfma_kernel<MAPS, 1>), dim3(grid), dim3(256), 0, st, a, bt);
+  else if (dk == 2) hipLaunchKernelGGL((paged_attn_mfma_kernel<MAPS, 2>), dim3(grid), dim3(256), 0, st, a, bt);
+  else if (dk == 3) hipLaunchKernelGGL((paged_attn_mfma_kernel<MAPS, 3>), dim3(grid), dim3(256), 0, st, a, bt);
+  else hipLaunchKernelGGL((paged_attn_mfma_kernel<MAPS, 4>), dim3(grid), dim3(256), 0, st, a, bt);
+}
+
 extern "C" int ragged_paged_attn_mfma(AttnArgs a, Batch bt, int maps, hipStream_t st) {
   if (bt.T <= 0 || a.H <= 0 || a.G <= 0 || a.H % a.G || !ragged_paged_attn_mfma_ok(a.d, a.vd)) return -1;
   if ((maps != 1 && maps != 2) || !a.tiles || a.n_tiles <= 0 || (int64_t)a.n_tiles * a.H > 0x7fffffff) return -1;
   const unsigned grid = (unsigned)(a.n_tiles * a.H);
-  if (maps == 2) hipLaunchKernelGGL((paged_attn_mfma_kernel<2>), dim3(grid), dim3(256), 0, st, a, bt);
-  else hipLaunchKernelGGL((paged_attn_mfma_kernel<1>), dim3(grid), dim3(256), 0, st, a, bt);
+  if (maps == 2) launch_mfma<2>(a, bt, grid, st);
+  else launch_mfma<1>(a, bt, grid, st);
   return RAGGED_LAUNCH_OK();
 }
