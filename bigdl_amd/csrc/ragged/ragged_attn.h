@@ -21,4 +21,8 @@ struct AttnArgs {
   int n_rows;
   const int* tiles;      // MFMA kernel: [n_tiles][2] = (sequence in the batch, first row of the tile inside its portion)
   int n_tiles;
+  int64_t ldv;           // elements between the value rows of neighbouring keys (vd, or the key row's length when the
+                         // values are the leading channels of the key rows and vpages == kpages)
+  int sink;              // 1: exp(sink_score) joins every row's normaliser (a key that all queries see and that has no value)
+  float sink_score;
 };

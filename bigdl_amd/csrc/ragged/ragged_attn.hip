@@ -105,7 +105,7 @@ __global__ __launch_bounds__(512) void paged_attn_kernel(AttnArgs a, Batch bt, i
     // values: lanes over channel pairs (lanes past vd re-read the last pair; their sums are never stored), keys past
     // the query are read from the page's last valid row and weigh 0
     const int nk = i - pg * PAGE + 1 < PAGE ? i - pg * PAGE + 1 : PAGE;
-    const T* vbase = V + (((int64_t)page * a.G + g) * PAGE) * a.vd;
+    const T* vbase = V + (((int64_t)page * a.G + g) * PAGE) * a.ldv;
     float va[U][VRP][2], vb[U][VRP][2];
     auto load_values = [&](float (&dst)[U][VRP][2], int j0) {
 #pragma unroll
@@ -115,10 +115,10 @@ __global__ __launch_bounds__(512) void paged_attn_kernel(AttnArgs a, Batch bt, i
         for (int v = 0; v < VRP; ++v) {
           const int c = 2 * lane + 128 * v;
           if (VEC) {
-            Vec<T>::load2(vbase + (int64_t)j * a.vd + (c < a.vd ? c : a.vd - 2), dst[u][v][0], dst[u][v][1]);
+            Vec<T>::load2(vbase + (int64_t)j * a.ldv + (c < a.vd ? c : a.vd - 2), dst[u][v][0], dst[u][v][1]);
           } else {
-            dst[u][v][0] = to_f(vbase[(int64_t)j * a.vd + (c < a.vd ? c : a.vd - 1)]);
-            dst[u][v][1] = to_f(vbase[(int64_t)j * a.vd + (c + 1 < a.vd ? c + 1 : a.vd - 1)]);
+            dst[u][v][0] = to_f(vbase[(int64_t)j * a.ldv + (c < a.vd ? c : a.vd - 1)]);
+            dst[u][v][1] = to_f(vbase[(int64_t)j * a.ldv + (c + 1 < a.vd ? c + 1 : a.vd - 1)]);
           }
         }
       }
@@ -268,10 +268,12 @@ __global__ __launch_bounds__(512) void paged_attn_kernel(AttnArgs a, Batch bt, i
     for (int mp = 0; mp < MAPS; ++mp) {
       float M = -1e30f, L = 0.f, w[8];
       for (int wv = 0; wv < nw; ++wv) M = fmaxf(M, part0[wv * wstride + r * pstride + mp]);
+      if (a.sink) M = fmaxf(M, a.sink_score);
       for (int wv = 0; wv < nw; ++wv) {
         w[wv] = __expf(part0[wv * wstride + r * pstride + mp] - M);
         L += w[wv] * part0[wv * wstride + r * pstride + MAPS + mp];
       }
+      if (a.sink) L += __expf(a.sink_score - M);
       const float coef = (mp == 0 ? 1.0f : -a.lambda) / L;
 #pragma unroll
       for (int v = 0; v < VRP; ++v) {
@@ -327,7 +329,7 @@ static void launch_one(AttnArgs a, Batch bt, int nrows, int coal, hipStream_t st
 template <typename T, int MAPS>
 static void launch_rows(AttnArgs a, Batch bt, int nrows, hipStream_t st, int* rc) {
   constexpr int N = Vec<T>::N;
-  const bool vec = (a.vd % 2 == 0) && (a.d % N == 0);
+  const bool vec = (a.vd % 2 == 0) && (a.d % N == 0) && (a.ldv % 2 == 0);
   const int vrp = a.vd <= 128 ? 1 : a.vd <= 256 ? 2 : 4;
   if (!vec || vrp == 4) {
     if (vrp == 1) launch_one<T, MAPS, false, 1, 1>(a, bt, nrows, 0, st, rc);
@@ -352,7 +354,7 @@ static void launch_rows(AttnArgs a, Batch bt, int nrows, hipStream_t st, int* rc
 
 extern "C" int ragged_paged_attn(AttnArgs a, Batch bt, int maps, int dtype, hipStream_t st) {
   if (bt.T <= 0 || a.H <= 0 || a.G <= 0 || a.H % a.G || a.d <= 0 || a.vd <= 0 || a.vd > 128 * MAX_VRP) return -1;
-  if (maps != 1 && maps != 2) return -1;
+  if ((maps != 1 && maps != 2) || a.ldv < a.vd) return -1;
   const int nrows = a.rows ? a.n_rows : bt.T;
   if (nrows <= 0 || (int64_t)nrows * a.H > 0x7fffffff) return -1;
   int rc = 0;

@@ -98,7 +98,7 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
   Frag vreg[4];
   auto page_of = [&](int o) { return pages[o < kept_pages ? o : pl + (o - kept_pages)]; };
   auto load_values = [&](int page) {
-    const bf16* vsrc = V + (((int64_t)page * a.G + gk) * PAGE + lane) * a.vd;
+    const bf16* vsrc = V + (((int64_t)page * a.G + gk) * PAGE + lane) * a.ldv;
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
       const int e0 = 8 * (4 * it + wave);
@@ -241,6 +241,15 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
   }
   if (!rowok) return;
   // ---- epilogue: combine the maps, per-head norm, gate; the lane holds channels 16 eb + 4 g4 + i of its query
+  if (a.sink) {                                              // one more term in every normaliser
+#pragma unroll
+    for (int mp = 0; mp < MAPS; ++mp) {
+      const float mnew = fmaxf(m[mp], a.sink_score), corr = __expf(m[mp] - mnew);
+      l[mp] = l[mp] * corr + __expf(a.sink_score - mnew);
+#pragma unroll
+      for (int eb = 0; eb < MF_NEB; ++eb) O[mp][eb] *= corr;
+    }
+  }
   const float c0 = 1.0f / l[0];
   const float c1 = MAPS == 2 ? a.lambda / l[MAPS - 1] : 0.f;
   float ss = 0.f;
@@ -286,6 +295,7 @@ static void launch_mfma(AttnArgs a, Batch bt, unsigned grid, hipStream_t st) {
 
 extern "C" int ragged_paged_attn_mfma(AttnArgs a, Batch bt, int maps, hipStream_t st) {
   if (bt.T <= 0 || a.H <= 0 || a.G <= 0 || a.H % a.G || !ragged_paged_attn_mfma_ok(a.d, a.vd)) return -1;
+  if (a.ldv < a.vd || a.ldv % 8) return -1;                  // value rows are read 16 bytes at a time
   if ((maps != 1 && maps != 2) || !a.tiles || a.n_tiles <= 0 || (int64_t)a.n_tiles * a.H > 0x7fffffff) return -1;
   const unsigned grid = (unsigned)(a.n_tiles * a.H);
   if (maps == 2) launch_mfma<2>(a, bt, grid, st);

@@ -1,0 +1,241 @@
+// Routed experts of the ragged engine: the router (32-bit softmax scores, group-limited choice of the best experts) and
+// the row-wise expert products that serve single decoded tokens and short portions, where every (row, chosen expert) pair
+// reads its expert's weights once.  Long portions run their experts as dense library products over rows sorted by expert
+// (models/ragged_engine.py); they share the router and the activation kernel with this path.
+#include "ragged_common.h"
+
+using namespace ragged;
+
+constexpr int MOE_MAX_E = 256;      // experts
+constexpr int MOE_SLOTS = MOE_MAX_E / 64;
+
+// Scores s = softmax(W_r x) over all experts in float (x may be the bfloat16 rounding of the normed stream).  Experts
+// form `groups` equal runs of neighbours; a group's score is its best expert's; the `top` best experts of the `keep` best
+// groups are chosen, best first, with weight s * scale (no renormalisation).  Ties go to the lower lane.
+// One workgroup of four wavefronts per row: the wavefronts share the router's rows, wavefront 0 chooses.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x, int64_t ldx, const float* __restrict__ wr,
+                                                        int* __restrict__ idx, float* __restrict__ wts, int D, int E, int groups,
+                                                        int keep, int top, float scale) {
+  __shared__ float z[MOE_MAX_E];
+  __shared__ float gbest[64];
+  const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const T* xr = x + (int64_t)t * ldx;
+  for (int e = wave; e < E; e += 4) {
+    const float* w = wr + (int64_t)e * D;
+    float acc = 0.f;
+    for (int c = lane; c < D; c += 64) acc += w[c] * to_f(xr[c]);
+    acc = wave_sum(acc);
+    if (lane == 0) z[e] = acc;
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  float s[MOE_SLOTS];
+  float mx = -1e30f;
+#pragma unroll
+  for (int k = 0; k < MOE_SLOTS; ++k) {
+    const int e = lane + 64 * k;
+    s[k] = e < E ? z[e] : -1e30f;
+    mx = fmaxf(mx, s[k]);
+  }
+  mx = wave_max(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < MOE_SLOTS; ++k) {
+    const int e = lane + 64 * k;
+    s[k] = e < E ? expf(s[k] - mx) : 0.f;
+    sum += s[k];
+  }
+  sum = wave_sum(sum);
+#pragma unroll
+  for (int k = 0; k < MOE_SLOTS; ++k) {
+    const int e = lane + 64 * k;
+    s[k] = s[k] / sum;
+    if (e < E) z[e] = s[k];
+  }
+  // (a wavefront's LDS requests are served in order: the scores written above are what is read below)
+  const int gsz = E / groups;
+  if (groups > 1 && keep < groups) {
+    float g = -1.f;
+    if (lane < groups)
+      for (int j = 0; j < gsz; ++j) g = fmaxf(g, z[lane * gsz + j]);
+    bool kept = false;
+    for (int it = 0; it < keep; ++it) {
+      const float best = wave_max(kept ? -1.f : g);
+      const unsigned long long who = __ballot(!kept && g == best && lane < groups);
+      if (lane == __ffsll((long long)who) - 1) kept = true;
+    }
+    gbest[lane] = kept ? 1.f : 0.f;
+#pragma unroll
+    for (int k = 0; k < MOE_SLOTS; ++k) {
+      const int e = lane + 64 * k;
+      if (e < E && gbest[e / gsz] == 0.f) s[k] = -1.f;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < MOE_SLOTS; ++k)
+    if (lane + 64 * k >= E) s[k] = -1.f;
+  for (int it = 0; it < top; ++it) {
+    float mine = s[0];
+    int at = 0;
+#pragma unroll
+    for (int k = 1; k < MOE_SLOTS; ++k)
+      if (s[k] > mine) { mine = s[k]; at = k; }
+    const float best = wave_max(mine);
+    const unsigned long long who = __ballot(mine == best);
+    if (lane == __ffsll((long long)who) - 1) {
+      idx[(int64_t)t * top + it] = lane + 64 * at;
+      wts[(int64_t)t * top + it] = best * scale;
+#pragma unroll
+      for (int k = 0; k < MOE_SLOTS; ++k)
+        if (k == at) s[k] = -2.f;
+    }
+  }
+}
+
+extern "C" int ragged_moe_route(const void* x, int64_t ldx, const float* wr, int* idx, float* wts, int64_t rows, int D, int E,
+                                int groups, int keep, int top, float scale, int dtype, hipStream_t st) {
+  if (rows <= 0 || rows > 0x7fffffff || D <= 0 || E <= 0 || E > MOE_MAX_E || groups <= 0 || groups > 64 || E % groups) return -1;
+  if (keep <= 0 || keep > groups || top <= 0 || top > keep * (E / groups)) return -1;
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((moe_route_kernel<T>), dim3((unsigned)rows), dim3(256), 0, st, (const T*)x, ldx, wr, idx,
+                                            wts, D, E, groups, keep, top, scale))
+  return RAGGED_LAUNCH_OK();
+}
+
+// relu(a)^2, elementwise
+template <typename T>
+__global__ __launch_bounds__(256) void relu2_kernel(const T* __restrict__ a, T* __restrict__ out, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const float v = fmaxf(to_f(a[i]), 0.f);
+    out[i] = from_f<T>(v * v);
+  }
+}
+
+extern "C" int ragged_relu2(const void* a, void* out, int64_t n, int dtype, hipStream_t st) {
+  if (n <= 0) return -1;
+  const unsigned grid = (unsigned)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((relu2_kernel<T>), dim3(grid), dim3(256), 0, st, (const T*)a, (T*)out, n))
+  return RAGGED_LAUNCH_OK();
+}
+
+// ---- row-wise expert products.  dot of a weight row with a vector held in LDS as floats, lanes striding 16 bytes
+template <typename T> struct WVec;
+template <> struct WVec<bf16> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void load(const bf16* p, float* o) {
+    const uint4 u = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      o[2 * i] = __uint_as_float(w[i] << 16);
+      o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+};
+template <> struct WVec<float> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ void load(const float* p, float* o) {
+    const float4 u = *reinterpret_cast<const float4*>(p);
+    o[0] = u.x; o[1] = u.y; o[2] = u.z; o[3] = u.w;
+  }
+};
+
+// partial dot products of R weight rows (row r at w + r * K) with xs[0 .. K), this lane's share; K % N == 0 and rows
+// 16-byte aligned when vec
+template <typename T, int R>
+__device__ __forceinline__ void rows_dot(const T* __restrict__ w, int64_t K, int nrows, const float* xs, bool vec, int lane,
+                                         float (&acc)[R]) {
+  constexpr int N = WVec<T>::N;
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = 0.f;
+  if (vec) {
+    for (int c = lane * N; c < K; c += 64 * N) {
+      float wv[R][N];
+#pragma unroll
+      for (int r = 0; r < R; ++r) WVec<T>::load(w + (int64_t)(r < nrows ? r : nrows - 1) * K + c, wv[r]);
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int e = 0; e < N; ++e) acc[r] += wv[r][e] * xs[c + e];
+    }
+  } else {
+    for (int c = lane; c < K; c += 64)
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[r] += to_f(w[(int64_t)(r < nrows ? r : nrows - 1) * K + c]) * xs[c];
+  }
+}
+
+constexpr int MOE_RW = 4;           // weight rows per wavefront and pass
+
+// A[(t, j), f] = relu(W_up[idx[t, j]][f, :] . x[t, :])^2.  Grid (rows * top, blocks of 4 * MOE_RW inner channels).
+template <typename T>
+__global__ __launch_bounds__(256) void moe_rows_up_kernel(const T* __restrict__ x, int64_t ldx, const int* __restrict__ idx,
+                                                          const T* __restrict__ w_up, T* __restrict__ A, int D, int ff, int top,
+                                                          int vec) {
+  extern __shared__ __attribute__((aligned(16))) float xs[];
+  const int pair = blockIdx.x, t = pair / top;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int c = threadIdx.x; c < D; c += 256) xs[c] = to_f(x[(int64_t)t * ldx + c]);
+  __syncthreads();
+  const int f0 = (blockIdx.y * 4 + wave) * MOE_RW;
+  if (f0 >= ff) return;
+  const int nrows = ff - f0 < MOE_RW ? ff - f0 : MOE_RW;
+  const T* w = w_up + ((int64_t)idx[pair] * ff + f0) * D;
+  float acc[MOE_RW];
+  rows_dot<T, MOE_RW>(w, D, nrows, xs, vec != 0, lane, acc);
+#pragma unroll
+  for (int r = 0; r < MOE_RW; ++r) {
+    const float v = fmaxf(wave_sum(acc[r]), 0.f);
+    if (lane == 0 && r < nrows) A[(int64_t)pair * ff + f0 + r] = from_f<T>(v * v);
+  }
+}
+
+// y[t, c] = base[t, c] + sum_j wts[t, j] * W_down[idx[t, j]][c, :] . A[(t, j), :].  Grid (rows, blocks of 4 * MOE_RW channels).
+template <typename T>
+__global__ __launch_bounds__(256) void moe_rows_down_kernel(const T* __restrict__ A, const int* __restrict__ idx,
+                                                            const float* __restrict__ wts, const T* __restrict__ w_dn,
+                                                            const T* __restrict__ base, T* __restrict__ y, int D, int ff, int top,
+                                                            int vec) {
+  extern __shared__ __attribute__((aligned(16))) float as[];
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int c0 = (blockIdx.y * 4 + wave) * MOE_RW;
+  const int nrows = c0 < D ? (D - c0 < MOE_RW ? D - c0 : MOE_RW) : 0;
+  float tot[MOE_RW];
+#pragma unroll
+  for (int r = 0; r < MOE_RW; ++r) tot[r] = 0.f;
+  for (int j = 0; j < top; ++j) {
+    __syncthreads();
+    for (int c = threadIdx.x; c < ff; c += 256) as[c] = to_f(A[((int64_t)t * top + j) * ff + c]);
+    __syncthreads();
+    if (nrows > 0) {
+      const T* w = w_dn + ((int64_t)idx[(int64_t)t * top + j] * D + c0) * ff;
+      float acc[MOE_RW];
+      rows_dot<T, MOE_RW>(w, ff, nrows, as, vec != 0, lane, acc);
+      const float wt = wts[(int64_t)t * top + j];
+#pragma unroll
+      for (int r = 0; r < MOE_RW; ++r) tot[r] += wt * wave_sum(acc[r]);
+    }
+  }
+  if (lane == 0)
+#pragma unroll
+    for (int r = 0; r < MOE_RW; ++r)
+      if (r < nrows) {
+        const int64_t o = (int64_t)t * D + c0 + r;
+        y[o] = from_f<T>(tot[r] + (base ? to_f(base[o]) : 0.f));
+      }
+}
+
+extern "C" int ragged_moe_rows(const void* x, int64_t ldx, const int* idx, const float* wts, const void* w_up, const void* w_dn,
+                               const void* base, void* A, void* y, int64_t rows, int D, int ff, int top, int dtype,
+                               hipStream_t st) {
+  if (rows <= 0 || D <= 0 || ff <= 0 || top <= 0 || rows * top > 0x7fffffff || D > 12288 || ff > 12288) return -1;
+  const int per = 4 * MOE_RW;
+  RAGGED_DISPATCH(dtype,
+    const int vu = D % WVec<T>::N == 0; const int vd = ff % WVec<T>::N == 0;
+    hipLaunchKernelGGL((moe_rows_up_kernel<T>), dim3((unsigned)(rows * top), (ff + per - 1) / per), dim3(256), D * sizeof(float), st,
+                       (const T*)x, ldx, idx, (const T*)w_up, (T*)A, D, ff, top, vu);
+    hipLaunchKernelGGL((moe_rows_down_kernel<T>), dim3((unsigned)rows, (D + per - 1) / per), dim3(256), ff * sizeof(float), st,
+                       (const T*)A, idx, wts, (const T*)w_dn, (const T*)base, (T*)y, D, ff, top, vd))
+  return RAGGED_LAUNCH_OK();
+}

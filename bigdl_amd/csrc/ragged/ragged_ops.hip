@@ -43,6 +43,45 @@ extern "C" int ragged_sum_group_norm(const float* x, const void* y, const float*
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// Sandwich form: x <- x + w_post * rmsnorm(y), then (w_next given) xa = w_next * rmsnorm(x) for the product that reads
+// the stream next.  One workgroup per row; x float in place, y and xa of type T.  Each thread re-reads only what it
+// wrote itself, so the passes need no barrier beyond those of the two sums.
+__device__ __forceinline__ float block_sum_256(float v, float* red) {
+  v = wave_sum(v);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void post_norm_add_kernel(float* __restrict__ x, const T* __restrict__ y,
+                                                            const float* __restrict__ w_post, const float* __restrict__ w_next,
+                                                            T* __restrict__ xa, int D, float eps) {
+  __shared__ float red[8];
+  const int64_t base = (int64_t)blockIdx.x * D;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < D; c += 256) { const float v = to_f(y[base + c]); ss += v * v; }
+  const float r1 = 1.0f / sqrtf(block_sum_256(ss, red) / (float)D + eps);
+  ss = 0.f;
+  for (int c = threadIdx.x; c < D; c += 256) {
+    const float v = x[base + c] + to_f(y[base + c]) * r1 * w_post[c];
+    x[base + c] = v;
+    ss += v * v;
+  }
+  if (!xa) return;
+  const float r2 = 1.0f / sqrtf(block_sum_256(ss, red + 4) / (float)D + eps);
+  for (int c = threadIdx.x; c < D; c += 256) xa[base + c] = from_f<T>(x[base + c] * r2 * w_next[c]);
+}
+
+extern "C" int ragged_post_norm_add(float* x, const void* y, const float* w_post, const float* w_next, void* xa, int64_t rows,
+                                    int D, float eps, int dtype, hipStream_t st) {
+  if (rows <= 0 || D <= 0 || rows > 0x7fffffff || !x || !y || !w_post || (xa && !w_next)) return -1;
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((post_norm_add_kernel<T>), dim3((unsigned)rows), dim3(256), 0, st, x, (const T*)y,
+                                            w_post, w_next, (T*)xa, D, eps))
+  return RAGGED_LAUNCH_OK();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
 // Short causal convolution over time per channel, then (optionally) RMS norm over groups of `gsize` channels with a
 // weight shared by all groups, then (optionally) rotation of the first `rot` channels of each group (pairs i, i + rot/2,
 // cosine and sine of the row's angles from a table made once per step), then a store into a dense float buffer or into
@@ -62,6 +101,9 @@ struct ConvHeadArgs {
   float* out_dense;       // [T, ngroups * gsize] or null
   void* pages;            // [num_pages, heads, PAGE, rowlen]
   int rowlen, heads;
+  int norm_n;             // leading channels of a group that the norm covers (0: all of them)
+  int rot0;               // first rotated channel of a group
+  int interleaved;        // 1: the pairs are neighbours (2 i, 2 i + 1) instead of (i, i + rot / 2)
 };
 
 template <typename T>
@@ -82,6 +124,7 @@ __global__ __launch_bounds__(256) void conv_head_kernel(ConvHeadArgs a, Batch bt
   }
   const T* P = (const T*)a.P;
   const T* S = (const T*)a.state;
+  const int nn = a.norm_n > 0 ? a.norm_n : a.gsize;
   float ss = 0.f;
   if (live) {
     for (int c = lane; c < a.gsize; c += 64) {
@@ -101,25 +144,27 @@ __global__ __launch_bounds__(256) void conv_head_kernel(ConvHeadArgs a, Batch bt
         v = to_f(P[(int64_t)t * a.ldp + a.col0 + f]);
       }
       buf[c] = v;
-      ss += v * v;
+      if (c < nn) ss += v * v;
     }
   }
   if (a.normw) {
     ss = wave_sum(ss);
-    const float r = 1.0f / sqrtf(ss / (float)a.gsize + a.eps);
+    const float r = 1.0f / sqrtf(ss / (float)nn + a.eps);
     if (live)
-      for (int c = lane; c < a.gsize; c += 64) buf[c] = buf[c] * r * a.normw[c];
+      for (int c = lane; c < nn; c += 64) buf[c] = buf[c] * r * a.normw[c];
   }
   __syncthreads();
   if (!live) return;
   const int half = a.rot >> 1;
   for (int c = lane; c < a.gsize; c += 64) {
     float v = buf[c];
-    if (c < a.rot) {
-      const int i = c < half ? c : c - half;
+    const int rc = c - a.rot0;
+    if (rc >= 0 && rc < a.rot) {
+      const bool first = a.interleaved ? !(rc & 1) : rc < half;
+      const int i = a.interleaved ? rc >> 1 : (first ? rc : rc - half), step = a.interleaved ? 1 : half;
       const float2 tr = *reinterpret_cast<const float2*>(a.cossin + ((int64_t)t * half + i) * 2);
       const float cs = tr.x, sn = tr.y;
-      v = c < half ? buf[c] * cs - buf[c + half] * sn : buf[c] * cs + buf[c - half] * sn;
+      v = first ? buf[c] * cs - buf[c + step] * sn : buf[c] * cs + buf[c - step] * sn;
     }
     const int f = grp * a.gsize + c;
     if (a.out_dense) {
@@ -135,7 +180,8 @@ __global__ __launch_bounds__(256) void conv_head_kernel(ConvHeadArgs a, Batch bt
 extern "C" int ragged_conv_head(ConvHeadArgs a, Batch bt, int dtype, hipStream_t st) {
   if (bt.T <= 0 || a.ngroups <= 0 || a.gsize <= 0 || a.gsize > 2048) return -1;
   if (a.cw && (a.taps < 1 || a.taps > 16 || (a.taps > 1 && !a.state))) return -1;
-  if (a.rot < 0 || (a.rot & 1) || a.rot > a.gsize || (a.rot && !a.cossin)) return -1;
+  if (a.rot < 0 || (a.rot & 1) || a.rot0 < 0 || a.rot0 + a.rot > a.gsize || (a.rot && !a.cossin)) return -1;
+  if (a.norm_n < 0 || a.norm_n > a.gsize) return -1;
   if (!a.out_dense && (!a.pages || a.rowlen <= 0 || (a.ngroups * a.gsize) % a.rowlen || a.heads * a.rowlen != a.ngroups * a.gsize))
     return -1;
   const int64_t items = (int64_t)bt.T * a.ngroups;
@@ -237,13 +283,16 @@ extern "C" int ragged_hgrn2_gates(const void* P, int64_t ldp, int q0, int f0, co
 constexpr int HG_DR = 32;
 constexpr int HG_SEG = HG_DR + 4;   // LDS floats per lane group and token (padding shifts the banks between groups)
 constexpr int HG_TBR = 64;          // TB * R <= this
-constexpr int HG_PRE = 2 * HG_TBR * HG_DR / 256;
-
-template <typename T>
+// GIN: the input's weights come from a third array, S <- diag(f_t) S + g_t v_t^T (mLSTM hands in f = its decay
+// repeated over the rows and g = its input gate times the key); otherwise g = 1 - f.
+template <typename T, bool GIN>
 __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* __restrict__ qf, const float* __restrict__ ff,
+                                                         const float* __restrict__ gf,
                                                          const T* __restrict__ P, int64_t ldp, int v0, float* __restrict__ state,
                                                          float* __restrict__ out, int H, int d, int vd, int R, int TB, Batch bt) {
-  extern __shared__ __attribute__((aligned(16))) float smem[];   // 2 x { q[TB][R][SEG], f[TB][R][SEG], v[TB][wcols] }
+  constexpr int NA = GIN ? 3 : 2;
+  constexpr int HG_PRE = NA * HG_TBR * HG_DR / 256;
+  extern __shared__ __attribute__((aligned(16))) float smem[];   // 2 x { q[TB][R][SEG], f[TB][R][SEG], (g,) v[TB][wcols] }
   const int b = blockIdx.z, h = blockIdx.y, tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int cols = 64 / R, wcols = 4 * cols;
@@ -254,7 +303,7 @@ __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* __restrict
   const int row0 = r * HG_DR;
   const int HD = H * d;
   const int qsz = TB * R * HG_SEG;                         // floats of q (and of f) in a buffer
-  const int bufsz = 2 * qsz + TB * wcols;
+  const int bufsz = NA * qsz + TB * wcols;
   float S[HG_DR];
   float* sp = state + (((int64_t)slot * H + h) * d) * vd;
   {
@@ -272,10 +321,11 @@ __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* __restrict
 #pragma unroll
     for (int u = 0; u < HG_PRE; ++u) {
       const int e = tid + 256 * u;
-      const int which = e >= nel, rem = which ? e - nel : e;
+      const int which = e / nel, rem = e - which * nel;
       const int tk = rem / (R * HG_DR), row = rem % (R * HG_DR);
-      float v = which ? 1.f : 0.f;                         // padding: f = 1, q = 0
-      if (e < 2 * nel && row < d && i0 + tk < n) v = (which ? ff : qf)[(int64_t)(start + i0 + tk) * HD + h * d + row];
+      float v = which == 1 ? 1.f : 0.f;                    // padding: f = 1, q = 0, g = 0
+      if (e < NA * nel && row < d && i0 + tk < n)
+        v = (which == 0 ? qf : which == 1 ? ff : gf)[(int64_t)(start + i0 + tk) * HD + h * d + row];
       pre[u] = v;
     }
 #pragma unroll
@@ -293,8 +343,8 @@ __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* __restrict
 #pragma unroll
     for (int u = 0; u < HG_PRE; ++u) {
       const int e = tid + 256 * u;
-      if (e < 2 * nel) {
-        const int which = e >= nel, rem = which ? e - nel : e;
+      if (e < NA * nel) {
+        const int which = e / nel, rem = e - which * nel;
         const int tk = rem / (R * HG_DR), row = rem % (R * HG_DR);
         buf[which * qsz + (tk * R + row / HG_DR) * HG_SEG + row % HG_DR] = pre[u];
       }
@@ -302,7 +352,7 @@ __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* __restrict
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int e = tid + 256 * u;
-      if (e < TB * wcols) buf[2 * qsz + e] = prev[u];
+      if (e < TB * wcols) buf[NA * qsz + e] = prev[u];
     }
   };
   if (n > 0) { fetch(0); stash(smem); }
@@ -316,18 +366,25 @@ __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* __restrict
     for (int tk = 0; tk < nt; ++tk) {
       const float4* q4 = reinterpret_cast<const float4*>(buf + (tk * R + r) * HG_SEG);
       const float4* f4 = reinterpret_cast<const float4*>(buf + qsz + (tk * R + r) * HG_SEG);
-      float qv[HG_DR], fv[HG_DR];
+      const float4* g4 = reinterpret_cast<const float4*>(buf + (NA - 1) * qsz + (tk * R + r) * HG_SEG);
+      float qv[HG_DR], fv[HG_DR], gv[HG_DR];
 #pragma unroll
       for (int k = 0; k < HG_DR / 4; ++k) {
         const float4 a = q4[k], c = f4[k];
         qv[4 * k] = a.x; qv[4 * k + 1] = a.y; qv[4 * k + 2] = a.z; qv[4 * k + 3] = a.w;
         fv[4 * k] = c.x; fv[4 * k + 1] = c.y; fv[4 * k + 2] = c.z; fv[4 * k + 3] = c.w;
+        if (GIN) {
+          const float4 e = g4[k];
+          gv[4 * k] = e.x; gv[4 * k + 1] = e.y; gv[4 * k + 2] = e.z; gv[4 * k + 3] = e.w;
+        } else {
+          gv[4 * k] = 1.0f - c.x; gv[4 * k + 1] = 1.0f - c.y; gv[4 * k + 2] = 1.0f - c.z; gv[4 * k + 3] = 1.0f - c.w;
+        }
       }
-      const float v = buf[2 * qsz + tk * wcols + lc];
+      const float v = buf[NA * qsz + tk * wcols + lc];
       float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int k = 0; k < HG_DR; ++k) {
-        S[k] = fv[k] * S[k] + (1.0f - fv[k]) * v;
+        S[k] = fv[k] * S[k] + gv[k] * v;
         acc[k & 3] += S[k] * qv[k];
       }
       const float tot = group_sum((acc[0] + acc[1]) + (acc[2] + acc[3]), R);
@@ -344,17 +401,23 @@ __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* __restrict
   }
 }
 
-extern "C" int ragged_hgrn2_scan(const float* qf, const float* ff, const void* P, int64_t ldp, int v0, float* state, float* out,
-                                 int H, int d, int vd, Batch bt, int dtype, hipStream_t st) {
+// gf null: the input's weight is 1 - f (HGRN2); otherwise the third gate array
+extern "C" int ragged_hgrn2_scan(const float* qf, const float* ff, const float* gf, const void* P, int64_t ldp, int v0,
+                                 float* state, float* out, int H, int d, int vd, Batch bt, int dtype, hipStream_t st) {
   if (bt.B <= 0 || H <= 0 || d <= 0 || vd <= 0 || d > HG_DR * 64) return -1;
   int R = 1;
   while (R * HG_DR < d) R <<= 1;
   const int wcols = 4 * (64 / R);
   int TB = HG_TBR / R < 16 ? HG_TBR / R : 16;
   if (TB * wcols > 4 * 256) TB = 4 * 256 / wcols;           // the value look-ahead holds 4 floats per thread
-  const size_t sm = 2 * (size_t)(2 * TB * R * HG_SEG + TB * wcols) * sizeof(float);
-  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((hgrn2_scan_kernel<T>), dim3((vd + wcols - 1) / wcols, H, bt.B), dim3(256), sm, st, qf,
-                                            ff, (const T*)P, ldp, v0, state, out, H, d, vd, R, TB, bt))
+  const int na = gf ? 3 : 2;
+  const size_t sm = 2 * (size_t)(na * TB * R * HG_SEG + TB * wcols) * sizeof(float);
+  const dim3 grid((vd + wcols - 1) / wcols, H, bt.B);
+  RAGGED_DISPATCH(dtype,
+    if (gf) hipLaunchKernelGGL((hgrn2_scan_kernel<T, true>), grid, dim3(256), sm, st, qf, ff, gf, (const T*)P, ldp, v0, state, out,
+                               H, d, vd, R, TB, bt);
+    else hipLaunchKernelGGL((hgrn2_scan_kernel<T, false>), grid, dim3(256), sm, st, qf, ff, gf, (const T*)P, ldp, v0, state, out,
+                            H, d, vd, R, TB, bt))
   return RAGGED_LAUNCH_OK();
 }
 

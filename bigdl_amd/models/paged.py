@@ -7,6 +7,8 @@ sequence (the tail of a short convolution's input, a recurrent layer's matrix st
 slots.  A layer declares what it keeps with a spec tuple:
 
     ("kv", heads, key_row, value_row)      pages  K [pages, heads, 64, key_row], V [pages, heads, 64, value_row]
+    ("k", heads, key_row)                  pages  K alone (a layer whose values are part of its key rows)
+    ("vector", size)                       slot   [slots, size]              float32
     ("tail", rows, channels)               slot   [slots, rows, channels]    activation type
     ("matrix", heads, rows, cols)          slot   [slots, heads, rows, cols] float32
 
@@ -35,6 +37,7 @@ class PagedStatePool:
         self.v: Dict[int, torch.Tensor] = {}
         self.tail: Dict[int, torch.Tensor] = {}
         self.matrix: Dict[int, torch.Tensor] = {}
+        self.vector: Dict[int, torch.Tensor] = {}
         for li, layer_specs in specs.items():
             for spec in layer_specs:
                 kind = spec[0]
@@ -42,6 +45,11 @@ class PagedStatePool:
                     _, heads, krow, vrow = spec
                     self.k[li] = torch.zeros(self.num_pages, heads, PAGE, krow, dtype=act_dtype, device=self.device)
                     self.v[li] = torch.zeros(self.num_pages, heads, PAGE, vrow, dtype=act_dtype, device=self.device)
+                elif kind == "k":
+                    _, heads, krow = spec
+                    self.k[li] = torch.zeros(self.num_pages, heads, PAGE, krow, dtype=act_dtype, device=self.device)
+                elif kind == "vector":
+                    self.vector[li] = torch.zeros(self.slots, spec[1], dtype=torch.float32, device=self.device)
                 elif kind == "tail":
                     _, rows, channels = spec
                     self.tail[li] = torch.zeros(self.slots, rows, channels, dtype=act_dtype, device=self.device)
@@ -91,4 +99,4 @@ class PagedStatePool:
         return sum(self.len_of.values())
 
     def nbytes(self) -> int:
-        return sum(t.numel() * t.element_size() for d in (self.k, self.v, self.tail, self.matrix) for t in d.values())
+        return sum(t.numel() * t.element_size() for d in (self.k, self.v, self.tail, self.matrix, self.vector) for t in d.values())

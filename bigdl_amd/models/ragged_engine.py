@@ -9,7 +9,8 @@ into arbitrary portions next to single decoded tokens run here instead:
   product runs once over all rows; the mixers read ``BatchMeta`` (row -> sequence, position, pages);
 * keys / values live in 64-token pages of a ``PagedStatePool``, per-sequence state in its slots;
 * the mixers are described by small dataclasses whose fields are the design's constants, so a new design is a new list
-  of them (``models/lipizen.py`` builds one from a ``config.json``);
+  of them (``models/lipizen.py`` and ``models/merusun.py`` build one from a ``config.json``);
+* two residual forms: the post-sum norm x <- norm(alpha x + f(x)), and the sandwich x <- x + norm_b(f(norm_a(x)));
 * matrix products are the library's (bf16 inputs with 32-bit accumulation, or plain float32), everything between them
   is ``ops/ragged.py``.
 """
@@ -50,6 +51,25 @@ class WindowAttention:
     keep_first: int = 0            # the first tokens stay visible behind the window
     gate: bool = False             # one sigmoid gate per head, from the mixer's input
     kv_from: Optional[int] = None  # read this layer's cache instead of projecting keys / values
+    bias: bool = False             # the q / k / v projections have biases
+    sink: Optional[float] = None   # score of a key without a value that every query sees: exp(sink) joins the normaliser
+
+
+@dataclass
+class LatentAttention:
+    """Attention over a compressed cache.  Per token one latent row c (``rank`` channels, RMS-normed with a weight) and
+    one rotated key part (``rot_dim`` channels) shared by all heads are kept; head h's keys are [W_uk,h c | rotated part],
+    its values W_uv,h c.  The engine folds W_uk into the queries and W_uv behind the weighted sum, so the kernel sees one
+    key/value head with key rows [c | rotated part] whose values are the rows' leading ``rank`` channels."""
+    heads: int
+    dim: int                       # unrotated channels of a head's queries and keys
+    rot_dim: int                   # rotated channels, after the unrotated ones
+    vdim: int
+    rank: int
+    scale: float
+    rot_dims: int = 0              # leading channels of the rotated part that turn (neighbouring pairs 2 i, 2 i + 1)
+    rot_base: float = 10000.0
+    window: int = 0
 
 
 @dataclass
@@ -61,11 +81,40 @@ class Hgrn2:
 
 
 @dataclass
+class Mlstm:
+    """Matrix memory with exponential gates held stable by a running maximum m (all per head, log gates i and f):
+    m' = max(f + m, i), S' = e^(f + m - m') S + e^(i - m') k v^T, n' likewise with k, o = S'^T q / (max(|n' . q|, e^-m') + tiny),
+    q scaled by dim^-1/2; gates are soft-capped, log f = logsigmoid(.).  Each head's output is divided by its root mean
+    square, weighted, and gated by a sigmoid of a projection of the mixer's input."""
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float
+    m_start: float = 0.0
+    den_floor: float = 1e-6
+
+
+@dataclass
 class ClampedGlu:
     """g = min(gate, limit), u = clamp(up, -limit, limit), y = g * sigmoid(slope * g) * (u + 1)"""
     ff: int
     limit: float
     slope: float = 1.702
+
+
+@dataclass
+class RoutedExperts:
+    """Mixture of two-matrix experts y = W_down act(W_up h), act = relu squared.  Scores are a softmax over all experts'
+    router logits (32-bit); experts come in ``groups`` equal runs of neighbours, a group scores as its best expert, and
+    the ``top`` best experts inside the ``keep`` best groups are used, weighted by score * ``scale`` (not renormalised).
+    ``shared_ff`` > 0: one more expert of that inner size that every token uses with weight 1."""
+    experts: int
+    top: int
+    ff: int
+    groups: int = 1
+    keep: int = 1
+    scale: float = 1.0
+    shared_ff: int = 0
 
 
 @dataclass
@@ -79,6 +128,8 @@ class RaggedConfig:
     residual_alpha: float = 1.0    # x <- norm(alpha * x + sublayer(x))
     logit_softcap: float = 0.0
     name: str = "ragged"
+    embed_scale: float = 1.0
+    block: str = "post_sum"        # "post_sum": x <- norm(alpha x + f(x)); "sandwich": x <- x + norm_b(f(norm_a(x)))
 
 
 @dataclass
@@ -96,6 +147,17 @@ class LayerTensors:
     o_norm: Optional[torch.Tensor] = None
     w_gu: Optional[torch.Tensor] = None      # [gate; up]
     w_down: Optional[torch.Tensor] = None
+    b_in: Optional[torch.Tensor] = None      # biases of the stacked input projections (zeros where there is none)
+    norm1b: Optional[torch.Tensor] = None    # sandwich form: norms behind the mixer and the feed-forward
+    norm2b: Optional[torch.Tensor] = None
+    w_uk: Optional[torch.Tensor] = None      # latent attention: [heads, dim, rank] and [heads, vdim, rank]
+    w_uv: Optional[torch.Tensor] = None
+    gate_bias: Optional[torch.Tensor] = None  # mLSTM: float [2 heads], input gates then forget gates
+    w_router: Optional[torch.Tensor] = None  # float [experts, width]
+    w_up: Optional[torch.Tensor] = None      # [experts, ff, width]
+    w_dn: Optional[torch.Tensor] = None      # [experts, width, ff]
+    w_sup: Optional[torch.Tensor] = None     # shared expert
+    w_sdn: Optional[torch.Tensor] = None
 
 
 def rotary_inv_freq(dims: int, base: float, factor: float) -> torch.Tensor:
@@ -139,8 +201,13 @@ class RaggedDecoder:
                     s.append(("kv", m.kv_heads, m.maps * m.dim, m.vdim))
                 if m.conv_taps > 1:
                     s.append(("tail", m.conv_taps - 1, self._conv_channels(m)))
+            elif isinstance(m, LatentAttention):
+                s.append(("k", 1, m.rank + m.rot_dim))          # values are the rows' leading channels
             elif isinstance(m, Hgrn2):
                 s.append(("matrix", m.heads, m.dim, m.vdim))
+            elif isinstance(m, Mlstm):
+                s.append(("matrix", m.heads, m.dim, m.vdim))
+                s.append(("vector", m.heads * (m.dim + 1)))     # per head: normaliser n[dim], then the running maximum
             specs[li] = s
         return specs
 
@@ -180,7 +247,62 @@ class RaggedDecoder:
         src = li if m.kv_from is None else m.kv_from
         return ops.paged_attn(q, pool.k[src], pool.v[src], meta, maps=m.maps, H=m.heads, G=m.kv_heads, d=m.dim, vd=m.vdim,
                               window=m.window, keep_first=m.keep_first, scale=m.scale, lam=m.lam, out_scale=m.out_scale,
-                              out_norm=m.out_norm, eps=eps, gate=P if m.gate else None, gate0=col)
+                              out_norm=m.out_norm, eps=eps, gate=P if m.gate else None, gate0=col, sink=m.sink)
+
+    def _latent(self, li, m: LatentAttention, lt: LayerTensors, P, meta):
+        """Scores of head h are q_h . [W_uk,h c | rotated part] = [W_uk,h^T q_h | rotated query part] . [c | rotated part]:
+        the queries are carried into the latent space (one batched product), the kernel attends over the cached rows with
+        one key/value head, and W_uv,h is applied to the weighted sum of latent rows afterwards."""
+        ops, pool, eps = self.ops, self.pool, self.cfg.norm_eps
+        T, H, hd = meta.T, m.heads, m.dim + m.rot_dim
+        qd = torch.empty(T, H * hd, dtype=torch.float32, device=self.device)
+        no_conv = dict(cw=None, taps=0, C=0, ch0=0, state=None)
+        ops.conv_head(P, 0, meta, ngroups=H, gsize=hd, normw=None, eps=eps, rot=m.rot_dims, rot0=m.dim, interleaved=True,
+                      inv_freq=lt.inv_freq, out_dense=qd, **no_conv)
+        ops.conv_head(P, H * hd, meta, ngroups=1, gsize=m.rank + m.rot_dim, normw=lt.k_norm, norm_n=m.rank, eps=eps,
+                      rot=m.rot_dims, rot0=m.rank, interleaved=True, inv_freq=lt.inv_freq, pages=pool.k[li], **no_conv)
+        q3 = qd.view(T, H, hd)
+        q = torch.empty(T, H, m.rank + m.rot_dim, dtype=torch.float32, device=self.device)
+        q[:, :, :m.rank] = torch.bmm(q3[:, :, :m.dim].to(self.act).transpose(0, 1), lt.w_uk).transpose(0, 1)
+        q[:, :, m.rank:] = q3[:, :, m.dim:]
+        o = ops.paged_attn(q.view(T, -1), pool.k[li], pool.k[li], meta, maps=1, H=H, G=1, d=m.rank + m.rot_dim, vd=m.rank,
+                           window=m.window, keep_first=0, scale=m.scale, lam=0.0, out_scale=1.0, out_norm=False, eps=eps)
+        return torch.bmm(o.view(T, H, m.rank).transpose(0, 1), lt.w_uv.transpose(1, 2)).transpose(0, 1).reshape(T, H * m.vdim)
+
+    def _mlstm(self, li, m: Mlstm, lt: LayerTensors, P, meta):
+        ops, pool = self.ops, self.pool
+        hd, hv = m.heads * m.dim, m.heads * m.vdim
+        # columns of P: q | k | v | output gate | input gates | forget gates
+        qf, ff, gf = ops.mlstm_prepare(P, 0, hd, 2 * hd + 2 * hv, lt.gate_bias, m.gate_cap, m.m_start, m.den_floor,
+                                       m.heads, m.dim, pool.vector[li], meta)
+        o = ops.hgrn2_scan(qf, ff, P, 2 * hd, pool.matrix[li], m.heads, m.dim, m.vdim, meta, gf=gf)
+        return ops.head_norm_gate(o, lt.o_norm, P, 2 * hd + hv, m.heads, m.vdim, self.cfg.norm_eps, self.act)
+
+    # rows per expert (on average) from which the experts run as dense products over their sorted rows; below, every
+    # (row, chosen expert) pair is served by the row-wise kernels, which read no more than the chosen experts' weights
+    moe_dense_rows = 16
+
+    def _experts(self, f: RoutedExperts, lt: LayerTensors, xa, meta):
+        ops = self.ops
+        idx, wts = ops.moe_route(xa, lt.w_router, f.groups, f.keep, f.top, f.scale)
+        base = None
+        if f.shared_ff:
+            base = F.linear(ops.relu2(F.linear(xa, lt.w_sup)), lt.w_sdn)
+        if meta.T * f.top < self.moe_dense_rows * f.experts:
+            return ops.moe_rows(xa, idx, wts, lt.w_up, lt.w_dn, base)
+        y = torch.zeros(meta.T, self.cfg.width, dtype=torch.float32, device=self.device) if base is None else base.float()
+        order = idx.view(-1).sort(stable=True)
+        counts = torch.bincount(order.values, minlength=f.experts).tolist()     # (the host learns the segment sizes)
+        pair = order.indices
+        rows, wsel = pair // f.top, wts.view(-1)[pair]
+        at = 0
+        for e, c in enumerate(counts):
+            if c:
+                r = rows[at:at + c]
+                out = F.linear(ops.relu2(F.linear(xa[r], lt.w_up[e])), lt.w_dn[e])
+                y.index_add_(0, r, out.float() * wsel[at:at + c, None])
+                at += c
+        return y.to(self.act)
 
     def _hgrn2(self, li, m: Hgrn2, lt: LayerTensors, P, meta):
         ops = self.ops
@@ -253,20 +375,34 @@ class RaggedDecoder:
         self.graph_replays += 1
         return ent["logits"].clone()
 
+    def _mixer(self, li, m, lt, P, meta):
+        if isinstance(m, WindowAttention):
+            return self._attention(li, m, lt, P, meta)
+        if isinstance(m, LatentAttention):
+            return self._latent(li, m, lt, P, meta)
+        if isinstance(m, Mlstm):
+            return self._mlstm(li, m, lt, P, meta)
+        return self._hgrn2(li, m, lt, P, meta)
+
     def _forward(self, meta, idt, rows, collect):
         cfg, ops = self.cfg, self.ops
         x = F.embedding(idt, self.embed).float()
-        xa = x.to(self.act)
-        for li, (m, mlp, lt) in enumerate(zip(cfg.mixers, cfg.mlps, self.layers)):
-            P = F.linear(xa, lt.w_in)
-            a = self._attention(li, m, lt, P, meta) if isinstance(m, WindowAttention) else self._hgrn2(li, m, lt, P, meta)
-            xa = ops.sum_group_norm(x, F.linear(a, lt.w_out), lt.norm1, cfg.norm_groups, cfg.residual_alpha, cfg.norm_eps, self.act)
-            if mlp is not None:
-                a = ops.clamped_glu(F.linear(xa, lt.w_gu), mlp.limit, mlp.slope)
-                xa = ops.sum_group_norm(x, F.linear(a, lt.w_down), lt.norm2, cfg.norm_groups, cfg.residual_alpha, cfg.norm_eps,
+        if cfg.embed_scale != 1.0:
+            x = x * cfg.embed_scale
+        if cfg.block == "sandwich":
+            self._sandwich_layers(x, meta, collect)
+        else:
+            xa = x.to(self.act)
+            for li, (m, mlp, lt) in enumerate(zip(cfg.mixers, cfg.mlps, self.layers)):
+                a = self._mixer(li, m, lt, F.linear(xa, lt.w_in, lt.b_in), meta)
+                xa = ops.sum_group_norm(x, F.linear(a, lt.w_out), lt.norm1, cfg.norm_groups, cfg.residual_alpha, cfg.norm_eps,
                                         self.act)
-            if collect is not None:
-                collect.append(x.clone())
+                if mlp is not None:
+                    a = ops.clamped_glu(F.linear(xa, lt.w_gu), mlp.limit, mlp.slope)
+                    xa = ops.sum_group_norm(x, F.linear(a, lt.w_down), lt.norm2, cfg.norm_groups, cfg.residual_alpha,
+                                            cfg.norm_eps, self.act)
+                if collect is not None:
+                    collect.append(x.clone())
         if not rows:
             return torch.empty(0, cfg.vocab, dtype=torch.float32, device=self.device)
         if rows == list(range(meta.T)):
@@ -279,6 +415,23 @@ class RaggedDecoder:
         if cfg.logit_softcap > 0:
             logits = torch.tanh(logits / cfg.logit_softcap) * cfg.logit_softcap
         return logits
+
+    def _sandwich_layers(self, x, meta, collect):
+        """x <- x + norm_b(f(norm_a(x))) for the mixer and the feed-forward of every layer; x float32, in place.  The norm
+        behind a sublayer, the residual sum and the norm in front of the next sublayer are one kernel."""
+        cfg, ops, eps = self.cfg, self.ops, self.cfg.norm_eps
+        n = len(self.layers)
+        xa = ops.row_norm(x, self.layers[0].norm1, eps, self.act) if n else None
+        for li, (m, mlp, lt) in enumerate(zip(cfg.mixers, cfg.mlps, self.layers)):
+            nxt = self.layers[li + 1].norm1 if li + 1 < n else None
+            a = self._mixer(li, m, lt, F.linear(xa, lt.w_in, lt.b_in), meta)
+            xa = ops.post_norm_add(x, F.linear(a, lt.w_out), lt.norm1b, nxt if mlp is None else lt.norm2, eps, self.act)
+            if isinstance(mlp, RoutedExperts):
+                xa = ops.post_norm_add(x, self._experts(mlp, lt, xa, meta), lt.norm2b, nxt, eps, self.act)
+            elif mlp is not None:
+                raise ValueError("the sandwich form has no such feed-forward yet")
+            if collect is not None:
+                collect.append(x.clone())
 
     # ------------------------------------------------------------------ generation
     @torch.no_grad()

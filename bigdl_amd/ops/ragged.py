@@ -63,7 +63,8 @@ class _ConvHeadArgs(ctypes.Structure):
                 ("taps", ctypes.c_int), ("C", ctypes.c_int), ("ch0", ctypes.c_int), ("state", ctypes.c_void_p),
                 ("ngroups", ctypes.c_int), ("gsize", ctypes.c_int), ("normw", ctypes.c_void_p), ("eps", ctypes.c_float),
                 ("rot", ctypes.c_int), ("cossin", ctypes.c_void_p), ("out_dense", ctypes.c_void_p),
-                ("pages", ctypes.c_void_p), ("rowlen", ctypes.c_int), ("heads", ctypes.c_int)]
+                ("pages", ctypes.c_void_p), ("rowlen", ctypes.c_int), ("heads", ctypes.c_int), ("norm_n", ctypes.c_int),
+                ("rot0", ctypes.c_int), ("interleaved", ctypes.c_int)]
 
 
 class _AttnArgs(ctypes.Structure):
@@ -72,7 +73,8 @@ class _AttnArgs(ctypes.Structure):
                 ("G", ctypes.c_int), ("d", ctypes.c_int), ("vd", ctypes.c_int), ("window", ctypes.c_int),
                 ("keep_first", ctypes.c_int), ("scale", ctypes.c_float), ("lam", ctypes.c_float),
                 ("out_scale", ctypes.c_float), ("out_norm", ctypes.c_int), ("eps", ctypes.c_float),
-                ("rows", ctypes.c_void_p), ("n_rows", ctypes.c_int), ("tiles", ctypes.c_void_p), ("n_tiles", ctypes.c_int)]
+                ("rows", ctypes.c_void_p), ("n_rows", ctypes.c_int), ("tiles", ctypes.c_void_p), ("n_tiles", ctypes.c_int),
+                ("ldv", ctypes.c_int64), ("sink", ctypes.c_int), ("sink_score", ctypes.c_float)]
 
 
 def lib():
@@ -87,7 +89,13 @@ def lib():
         L.ragged_conv_state.argtypes = [vp, i64, ci, vp, ci, ci, _Batch, ci, vp]
         L.ragged_clamped_glu.argtypes = [vp, vp, i64, ci, cf, cf, ci, vp]
         L.ragged_hgrn2_gates.argtypes = [vp, i64, ci, ci, vp, vp, vp, vp, i64, ci, ci, vp]
-        L.ragged_hgrn2_scan.argtypes = [vp, vp, vp, i64, ci, vp, vp, ci, ci, ci, _Batch, ci, vp]
+        L.ragged_hgrn2_scan.argtypes = [vp, vp, vp, vp, i64, ci, vp, vp, ci, ci, ci, _Batch, ci, vp]
+        L.ragged_post_norm_add.argtypes = [vp, vp, vp, vp, vp, i64, ci, cf, ci, vp]
+        L.ragged_mlstm_prepare.argtypes = [vp, i64, ci, ci, ci, vp, cf, cf, cf, vp, vp, vp, vp, ci, ci, _Batch, ci, vp]
+        L.ragged_head_norm_gate.argtypes = [vp, vp, vp, i64, ci, vp, i64, ci, ci, cf, ci, vp]
+        L.ragged_moe_route.argtypes = [vp, i64, vp, vp, vp, i64, ci, ci, ci, ci, ci, cf, ci, vp]
+        L.ragged_relu2.argtypes = [vp, vp, i64, ci, vp]
+        L.ragged_moe_rows.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, i64, ci, ci, ci, ci, vp]
         L.ragged_hgrn2_chunk_decay.argtypes = [vp, vp, vp, ci, ci, vp]
         L.ragged_hgrn2_chunk_combine.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, vp]
         L.ragged_row_norm.argtypes = [vp, vp, vp, i64, ci, cf, ci, vp]
@@ -264,7 +272,7 @@ class HipOps:
         return xa
 
     def conv_head(self, P, col0, meta, *, cw, taps, C, ch0, state, ngroups, gsize, normw, eps, rot, inv_freq,
-                  out_dense=None, pages=None):
+                  out_dense=None, pages=None, norm_n=None, rot0=0, interleaved=False):
         _act(P, state, pages)
         _f32(cw, normw, inv_freq, out_dense)
         if P.dim() != 2 or P.shape[0] != meta.T or col0 < 0 or col0 + ngroups * gsize > P.shape[1]:
@@ -281,13 +289,13 @@ class HipOps:
             a.state = None if state is None else state.data_ptr()
         a.ngroups, a.gsize, a.eps = ngroups, gsize, eps
         if normw is not None:
-            if normw.numel() != gsize:
-                raise ValueError("norm weight must have the group's size")
-            a.normw = normw.data_ptr()
+            if normw.numel() != (gsize if norm_n is None else norm_n) or not 0 < normw.numel() <= gsize:
+                raise ValueError("norm weight must have the size of the group's normed part")
+            a.normw, a.norm_n = normw.data_ptr(), normw.numel()
         if rot:
-            if inv_freq.numel() != rot // 2:
-                raise ValueError("one frequency per rotated pair")
-            a.rot, a.cossin = rot, meta.cossin(inv_freq).data_ptr()
+            if inv_freq.numel() != rot // 2 or rot % 2 or rot0 < 0 or rot0 + rot > gsize:
+                raise ValueError("one frequency per rotated pair, pairs inside the group")
+            a.rot, a.cossin, a.rot0, a.interleaved = rot, meta.cossin(inv_freq).data_ptr(), rot0, int(bool(interleaved))
         if out_dense is not None:
             if out_dense.shape != (meta.T, ngroups * gsize):
                 raise ValueError("dense output shape")
@@ -330,17 +338,20 @@ class HipOps:
                                      ff.data_ptr(), rows, HD, _DT[P.dtype], _stream()), "hgrn2_gates")
         return qf, ff
 
-    def hgrn2_scan(self, qf, ff, P, v0, state, H, d, vd, meta):
-        _f32(qf, ff, state)
+    def hgrn2_scan(self, qf, ff, P, v0, state, H, d, vd, meta, gf=None):
+        """S <- diag(f) S + g v^T, o = S^T q per head; g = 1 - f unless ``gf`` gives it."""
+        _f32(qf, ff, state, gf)
         _act(P)
         if qf.shape != (meta.T, H * d) or ff.shape != qf.shape or v0 + H * vd > P.shape[1] or P.shape[0] != meta.T \
-                or state.shape[1:] != (H, d, vd) or max(s[0] for s in meta.seqs) >= state.shape[0]:
+                or state.shape[1:] != (H, d, vd) or max(s[0] for s in meta.seqs) >= state.shape[0] \
+                or (gf is not None and gf.shape != qf.shape):
             raise ValueError("recurrent state / gates do not fit")
         out = torch.empty(meta.T, H * vd, dtype=torch.float32, device=P.device)
         L, dt, st = lib(), _DT[P.dtype], _stream()
+        g = None if gf is None else gf.data_ptr()
         longest = max(n for _, _, n, _ in meta.seqs)
         if longest < 2 * self.scan_chunk:
-            _ok(L.ragged_hgrn2_scan(qf.data_ptr(), ff.data_ptr(), P.data_ptr(), P.stride(0), v0, state.data_ptr(),
+            _ok(L.ragged_hgrn2_scan(qf.data_ptr(), ff.data_ptr(), g, P.data_ptr(), P.stride(0), v0, state.data_ptr(),
                                     out.data_ptr(), H, d, vd, meta.c(), dt, st), "hgrn2_scan")
             return out
         # long portions: chunks scanned side by side from zero, chunk-start states chained, chunks scanned again from them
@@ -351,13 +362,13 @@ class HipOps:
 
         def chunk_batch(past):
             return _Batch(None, None, cstart.data_ptr(), past.data_ptr(), cid.data_ptr(), None, meta.T, nc, 0)
-        _ok(L.ragged_hgrn2_scan(qf.data_ptr(), ff.data_ptr(), P.data_ptr(), P.stride(0), v0, local.data_ptr(), out.data_ptr(),
+        _ok(L.ragged_hgrn2_scan(qf.data_ptr(), ff.data_ptr(), g, P.data_ptr(), P.stride(0), v0, local.data_ptr(), out.data_ptr(),
                                 H, d, vd, chunk_batch(zeros), dt, st), "hgrn2_scan (chunks from zero)")
         _ok(L.ragged_hgrn2_chunk_decay(ff.data_ptr(), cstart.data_ptr(), decay.data_ptr(), nc, H * d, st), "hgrn2_chunk_decay")
         _ok(L.ragged_hgrn2_chunk_combine(state.data_ptr(), local.data_ptr(), decay.data_ptr(), begin.data_ptr(), cfirst.data_ptr(),
                                          meta.seq_past.data_ptr(), meta.seq_slot.data_ptr(), meta.B, H, d, vd, st),
             "hgrn2_chunk_combine")
-        _ok(L.ragged_hgrn2_scan(qf.data_ptr(), ff.data_ptr(), P.data_ptr(), P.stride(0), v0, begin.data_ptr(), out.data_ptr(),
+        _ok(L.ragged_hgrn2_scan(qf.data_ptr(), ff.data_ptr(), g, P.data_ptr(), P.stride(0), v0, begin.data_ptr(), out.data_ptr(),
                                 H, d, vd, chunk_batch(ones), dt, st), "hgrn2_scan (chunks from their start states)")
         slots = torch.tensor([s[0] for s in meta.seqs], dtype=torch.int64, device=P.device)
         state[slots] = begin[torch.tensor(last, dtype=torch.int64, device=P.device)]     # every sequence's end state
@@ -374,13 +385,16 @@ class HipOps:
         return out
 
     def paged_attn(self, q, kpages, vpages, meta, *, maps, H, G, d, vd, window, keep_first, scale, lam, out_scale, out_norm,
-                   eps, gate=None, gate0=0):
+                   eps, gate=None, gate0=0, sink=None):
+        """``vpages`` may be ``kpages`` itself: the values are then the leading ``vd`` channels of the key rows."""
         _f32(q)
         _act(kpages, vpages, gate)
         _page_check(meta, kpages)
         _page_check(meta, vpages)
-        if q.shape != (meta.T, H * maps * d) or kpages.shape[1:] != (G, PAGE, maps * d) or vpages.shape[1:] != (G, PAGE, vd) \
-                or kpages.dtype != vpages.dtype or kpages.shape[0] != vpages.shape[0]:
+        shared = vpages.data_ptr() == kpages.data_ptr()
+        if q.shape != (meta.T, H * maps * d) or kpages.shape[1:] != (G, PAGE, maps * d) or kpages.dtype != vpages.dtype \
+                or kpages.shape[0] != vpages.shape[0] or not q.is_contiguous() \
+                or (vpages.shape[1:] != (G, PAGE, vd) and not (shared and vd <= maps * d)):
             raise ValueError("queries / cache pages do not fit the head layout")
         out = torch.empty(meta.T, H * vd, dtype=kpages.dtype, device=q.device)
         a = _AttnArgs()
@@ -391,7 +405,10 @@ class HipOps:
             a.gate, a.ldg, a.gate0 = gate.data_ptr(), gate.stride(0), gate0
         a.H, a.G, a.d, a.vd, a.window, a.keep_first = H, G, d, vd, window, keep_first
         a.scale, a.lam, a.out_scale, a.out_norm, a.eps = scale, lam, out_scale, int(out_norm), eps
-        if kpages.dtype == torch.bfloat16 and self.mfma and lib().ragged_paged_attn_mfma_ok(d, vd):
+        a.ldv = vpages.shape[3]
+        if sink is not None:
+            a.sink, a.sink_score = 1, float(sink)
+        if kpages.dtype == torch.bfloat16 and self.mfma and lib().ragged_paged_attn_mfma_ok(d, vd) and a.ldv % 8 == 0:
             # long portions on the matrix cores, single tokens and short portions row by row
             tiles, n_tiles, rows, n_rows = meta.attn_split(self.mfma_min_rows)
             if n_tiles:
@@ -403,6 +420,85 @@ class HipOps:
             return out
         _ok(lib().ragged_paged_attn(a, meta.c(), maps, _DT[kpages.dtype], _stream()), "paged_attn")
         return out
+
+    def post_norm_add(self, x, y, w_post, w_next, eps, act):
+        """x <- x + w_post * rmsnorm(y) in place; returns w_next * rmsnorm(x) as ``act`` (None without ``w_next``)."""
+        _f32(x, w_post, w_next)
+        _act(y)
+        rows, D = x.shape
+        if y.shape != x.shape or not y.is_contiguous() or y.dtype != act or w_post.numel() != D \
+                or (w_next is not None and w_next.numel() != D):
+            raise ValueError("sublayer output / norm weights do not fit the stream")
+        xa = None if w_next is None else torch.empty(rows, D, dtype=act, device=x.device)
+        _ok(lib().ragged_post_norm_add(x.data_ptr(), y.data_ptr(), w_post.data_ptr(), None if w_next is None else w_next.data_ptr(),
+                                       None if xa is None else xa.data_ptr(), rows, D, eps, _DT[act], _stream()), "post_norm_add")
+        return xa
+
+    def relu2(self, A):
+        _act(A)
+        if not A.is_contiguous():
+            raise ValueError("contiguous activations expected")
+        out = torch.empty_like(A)
+        if A.numel():
+            _ok(lib().ragged_relu2(A.data_ptr(), out.data_ptr(), A.numel(), _DT[A.dtype], _stream()), "relu2")
+        return out
+
+    def head_norm_gate(self, o, w, P, g0, H, vd, eps, act):
+        _f32(o, w)
+        _act(P)
+        T = o.shape[0]
+        if o.shape != (T, H * vd) or w.numel() != H * vd or P.shape[0] != T or g0 + H * vd > P.shape[1] or P.dtype != act:
+            raise ValueError("head outputs / gate columns do not fit")
+        out = torch.empty(T, H * vd, dtype=act, device=o.device)
+        _ok(lib().ragged_head_norm_gate(o.data_ptr(), w.data_ptr(), P.data_ptr(), P.stride(0), g0, out.data_ptr(), T, H, vd, eps,
+                                        _DT[act], _stream()), "head_norm_gate")
+        return out
+
+    def mlstm_prepare(self, P, q0, k0, i0, gate_bias, cap, m_start, den_floor, H, d, vec, meta):
+        """The scalar part of the mLSTM recurrence over this step's rows; returns (q / denominator, decay, input gate
+        times key), each float [T, H d], for the matrix scan.  ``vec`` [slots, H (d + 1)] carries n and m."""
+        _act(P)
+        _f32(gate_bias, vec)
+        if P.shape[0] != meta.T or max(q0, k0) + H * d > P.shape[1] or i0 + 2 * H > P.shape[1] or gate_bias.numel() != 2 * H \
+                or vec.shape[1] != H * (d + 1) or max(s[0] for s in meta.seqs) >= vec.shape[0]:
+            raise ValueError("gate columns / state slots do not fit")
+        qf = torch.empty(meta.T, H * d, dtype=torch.float32, device=P.device)
+        ff, gf = torch.empty_like(qf), torch.empty_like(qf)
+        _ok(lib().ragged_mlstm_prepare(P.data_ptr(), P.stride(0), q0, k0, i0, gate_bias.data_ptr(), cap, m_start, den_floor,
+                                       vec.data_ptr(), qf.data_ptr(), ff.data_ptr(), gf.data_ptr(), H, d, meta.c(), _DT[P.dtype],
+                                       _stream()), "mlstm_prepare")
+        return qf, ff, gf
+
+    def moe_route(self, xa, w_router, groups, keep, top, scale):
+        _act(xa)
+        _f32(w_router)
+        T, D = xa.shape
+        E = w_router.shape[0]
+        if w_router.shape[1] != D:
+            raise ValueError("router rows do not fit the stream")
+        idx = torch.empty(T, top, dtype=torch.int32, device=xa.device)
+        wts = torch.empty(T, top, dtype=torch.float32, device=xa.device)
+        _ok(lib().ragged_moe_route(xa.data_ptr(), xa.stride(0), w_router.data_ptr(), idx.data_ptr(), wts.data_ptr(), T, D, E, groups,
+                                   keep, top, scale, _DT[xa.dtype], _stream()), "moe_route")
+        return idx, wts
+
+    def moe_rows(self, xa, idx, wts, w_up, w_dn, base):
+        """y = base + sum over a row's chosen experts of weight * W_down relu(W_up x)^2, every pair served on its own."""
+        _act(xa, w_up, w_dn, base)
+        _f32(wts)
+        T, D = xa.shape
+        E, ff, top = w_up.shape[0], w_up.shape[1], idx.shape[1]
+        if w_up.shape != (E, ff, D) or w_dn.shape != (E, D, ff) or not w_up.is_contiguous() or not w_dn.is_contiguous() \
+                or w_up.dtype != xa.dtype or w_dn.dtype != xa.dtype or idx.shape != (T, top) or wts.shape != (T, top) \
+                or idx.dtype != torch.int32 or not idx.is_contiguous() \
+                or (base is not None and (base.shape != (T, D) or base.dtype != xa.dtype or not base.is_contiguous())):
+            raise ValueError("expert weights / choices do not fit")
+        A = torch.empty(T * top, ff, dtype=xa.dtype, device=xa.device)
+        y = torch.empty(T, D, dtype=xa.dtype, device=xa.device)
+        _ok(lib().ragged_moe_rows(xa.data_ptr(), xa.stride(0), idx.data_ptr(), wts.data_ptr(), w_up.data_ptr(), w_dn.data_ptr(),
+                                  None if base is None else base.data_ptr(), A.data_ptr(), y.data_ptr(), T, D, ff, top,
+                                  _DT[xa.dtype], _stream()), "moe_rows")
+        return y
 
 
 class TorchOps:
@@ -438,17 +534,24 @@ class TorchOps:
         return out
 
     def conv_head(self, P, col0, meta, *, cw, taps, C, ch0, state, ngroups, gsize, normw, eps, rot, inv_freq,
-                  out_dense=None, pages=None):
+                  out_dense=None, pages=None, norm_n=None, rot0=0, interleaved=False):
         width = ngroups * gsize
         v = self._segment(P, col0, meta, cw, taps, C, ch0, state, width).view(meta.T, ngroups, gsize)
         if normw is not None:
-            v = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps) * normw
+            nn = gsize if norm_n is None else norm_n
+            u = v[..., :nn]
+            v = torch.cat([u / torch.sqrt(u.pow(2).mean(-1, keepdim=True) + eps) * normw, v[..., nn:]], -1)
         if rot:
             half = rot // 2
             ang = meta.tok_pos.to(P.device).float()[:, None] * inv_freq[None]
             c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
-            a, b2 = v[..., :half], v[..., half:rot]
-            v = torch.cat([a * c - b2 * s, b2 * c + a * s, v[..., rot:]], -1)
+            if interleaved:
+                a, b2 = v[..., rot0:rot0 + rot:2], v[..., rot0 + 1:rot0 + rot:2]
+                turned = torch.stack([a * c - b2 * s, b2 * c + a * s], -1).flatten(-2)
+            else:
+                a, b2 = v[..., rot0:rot0 + half], v[..., rot0 + half:rot0 + rot]
+                turned = torch.cat([a * c - b2 * s, b2 * c + a * s], -1)
+            v = torch.cat([v[..., :rot0], turned, v[..., rot0 + rot:]], -1)
         v = v.reshape(meta.T, width)
         if out_dense is not None:
             out_dense.copy_(v)
@@ -480,14 +583,14 @@ class TorchOps:
         f = lower + (1 - lower) * torch.sigmoid(P[:, f0:f0 + HD].float() + fb)
         return q * torch.sigmoid(q), f
 
-    def hgrn2_scan(self, qf, ff, P, v0, state, H, d, vd, meta):
+    def hgrn2_scan(self, qf, ff, P, v0, state, H, d, vd, meta, gf=None):
         out = torch.empty(meta.T, H * vd, dtype=torch.float32, device=P.device)
         for b, (slot, past, n, _) in enumerate(meta.seqs):
             S = state[slot].clone() if past > 0 else torch.zeros_like(state[slot])
             for i in range(n):
                 t = meta.start[b] + i
                 f = ff[t].view(H, d, 1)
-                S = f * S + (1 - f) * P[t, v0:v0 + H * vd].float().view(H, 1, vd)
+                S = f * S + (1 - f if gf is None else gf[t].view(H, d, 1)) * P[t, v0:v0 + H * vd].float().view(H, 1, vd)
                 out[t] = (S * qf[t].view(H, d, 1)).sum(1).reshape(-1)
             state[slot] = S
         return out
@@ -497,14 +600,14 @@ class TorchOps:
         return (v if w is None else v * w).to(act)
 
     def paged_attn(self, q, kpages, vpages, meta, *, maps, H, G, d, vd, window, keep_first, scale, lam, out_scale, out_norm,
-                   eps, gate=None, gate0=0):
+                   eps, gate=None, gate0=0, sink=None):
         out = torch.empty(meta.T, H * vd, dtype=torch.float32, device=q.device)
         q = q.view(meta.T, H, maps, d)
         for b, (slot, past, n, pg) in enumerate(meta.seqs):
             L = past + n
             idx = torch.tensor(pg, dtype=torch.long, device=q.device)
             k = kpages[idx].float().permute(1, 0, 2, 3).reshape(G, -1, maps, d)[:, :L]       # [G, L, maps, d]
-            v = vpages[idx].float().permute(1, 0, 2, 3).reshape(G, -1, vd)[:, :L]
+            v = vpages[idx][..., :vd].float().permute(1, 0, 2, 3).reshape(G, -1, vd)[:, :L]
             i = torch.arange(past, L, device=q.device)[:, None]
             j = torch.arange(L, device=q.device)[None]
             vis = j <= i
@@ -515,7 +618,14 @@ class TorchOps:
             o = None
             for mp in range(maps):
                 s = torch.einsum("thd,hld->htl", qs[:, :, mp], k[:, :, mp].repeat_interleave(rep, 0)) * scale
-                a = torch.softmax(s.masked_fill(~vis, float("-inf")), -1) @ v.repeat_interleave(rep, 0)   # [H, n, vd]
+                s = s.masked_fill(~vis, float("-inf"))
+                if sink is None:
+                    w = torch.softmax(s, -1)
+                else:                                     # one more score in the normaliser, no value behind it
+                    top = s.max(-1, keepdim=True).values.clamp(min=sink)
+                    w = torch.exp(s - top)
+                    w = w / (w.sum(-1, keepdim=True) + torch.exp(sink - top))
+                a = w @ v.repeat_interleave(rep, 0)       # [H, n, vd]
                 o = a if mp == 0 else o - lam * a
             o = o.permute(1, 0, 2)
             if out_norm:
@@ -524,6 +634,61 @@ class TorchOps:
         if gate is not None:
             out = (out.view(meta.T, H, vd) * torch.sigmoid(gate[:, gate0:gate0 + H].float())[:, :, None]).view(meta.T, H * vd)
         return out.to(kpages.dtype)
+
+    def post_norm_add(self, x, y, w_post, w_next, eps, act):
+        v = y.float()
+        x += v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w_post
+        if w_next is None:
+            return None
+        return (x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w_next).to(act)
+
+    def relu2(self, A):
+        return torch.relu(A.float()).pow(2).to(A.dtype)
+
+    def head_norm_gate(self, o, w, P, g0, H, vd, eps, act):
+        v = o.view(-1, H, vd)
+        v = (v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)).reshape(-1, H * vd)
+        return (v * w * torch.sigmoid(P[:, g0:g0 + H * vd].float())).to(act)
+
+    def mlstm_prepare(self, P, q0, k0, i0, gate_bias, cap, m_start, den_floor, H, d, vec, meta):
+        T = meta.T
+        q = P[:, q0:q0 + H * d].float().view(T, H, d) * d ** -0.5
+        k = P[:, k0:k0 + H * d].float().view(T, H, d)
+        gi = cap * torch.tanh((P[:, i0:i0 + H].float() + gate_bias[:H]) / cap)
+        gfo = F.logsigmoid(cap * torch.tanh((P[:, i0 + H:i0 + 2 * H].float() + gate_bias[H:]) / cap))
+        qf, ff, gf = torch.empty(T, H, d), torch.empty(T, H, d), torch.empty(T, H, d)
+        for b, (slot, past, n, _) in enumerate(meta.seqs):
+            st = vec[slot].view(H, d + 1)
+            nv = st[:, :d].clone() if past > 0 else torch.zeros(H, d)
+            m = st[:, d].clone() if past > 0 else torch.full((H,), float(m_start))
+            for i in range(n):
+                t = meta.start[b] + i
+                m2 = torch.maximum(gfo[t] + m, gi[t])
+                a, bb = torch.exp(gfo[t] + m - m2), torch.exp(gi[t] - m2)
+                nv = a[:, None] * nv + bb[:, None] * k[t]
+                m = m2
+                den = torch.maximum((nv * q[t]).sum(-1).abs(), torch.exp(-m)) + den_floor
+                qf[t], ff[t], gf[t] = q[t] / den[:, None], a[:, None].expand(H, d), bb[:, None] * k[t]
+            st[:, :d], st[:, d] = nv, m
+        return qf.view(T, -1), ff.reshape(T, -1), gf.view(T, -1)
+
+    def moe_route(self, xa, w_router, groups, keep, top, scale):
+        s = torch.softmax(xa.float() @ w_router.t(), -1)
+        E = s.shape[1]
+        best = s.view(-1, groups, E // groups).max(-1).values
+        kept = torch.zeros_like(best, dtype=torch.bool)
+        kept.scatter_(1, best.topk(keep, -1).indices, True)
+        idx = s.masked_fill(~kept.repeat_interleave(E // groups, 1), -1.0).topk(top, -1).indices
+        return idx.to(torch.int32), s.gather(1, idx) * scale
+
+    def moe_rows(self, xa, idx, wts, w_up, w_dn, base):
+        y = torch.zeros(xa.shape[0], w_dn.shape[1]) if base is None else base.float().clone()
+        for t in range(xa.shape[0]):
+            for j in range(idx.shape[1]):
+                e = int(idx[t, j])
+                a = torch.relu(w_up[e].float() @ xa[t].float()).pow(2).to(xa.dtype)
+                y[t] += wts[t, j] * (w_dn[e].float() @ a.float())
+        return y.to(xa.dtype)
 
 
 def ops_for(device) -> object:
