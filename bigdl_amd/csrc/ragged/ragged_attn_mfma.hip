@@ -279,6 +279,224 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Wide rows: key rows of up to 32 DK channels and values of up to 16 NEB channels (one score map), as the latent
+// attention has them after its queries are carried into the latent space (keys [latent row | rotated part], values the
+// latent row).  Same tile, same transposed scores, same softmax and same two-term weights as above; what differs is
+// where the operands live: the output tile alone takes up to 128 registers, so K fragments are not held a page ahead but
+// come from memory a few 32-channel steps at a time (the four wavefronts of a workgroup read the same page, so three of
+// four reads hit the CU's cache), and the value tile is brought in and transposed 128 channels at a time.
+template <int DK, int NEB>
+__global__ __launch_bounds__(256) void paged_attn_mfma_wide_kernel(AttnArgs a, Batch bt) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t vt[];                   // V^T [16 NEB][PAGE (+ pad)]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int lq = lane & 15, g4 = lane >> 4;
+  const int tile = blockIdx.x / a.H, h = blockIdx.x % a.H;
+  const int b = a.tiles[2 * tile], row0 = a.tiles[2 * tile + 1];
+  const int start = bt.seq_start[b], n = bt.seq_start[b + 1] - start, past = bt.seq_past[b];
+  const int gk = h / (a.H / a.G);
+  const int neb = a.vd / 16;
+  const int nrows = n - row0 < 64 ? n - row0 : 64;
+  const int myrow = row0 + 16 * wave + lq;
+  const bool rowok = 16 * wave + lq < nrows;
+  const int qpos = rowok ? past + myrow : -1;
+  const int64_t t = start + (rowok ? myrow : row0);
+
+  Frag qf[DK];
+#pragma unroll
+  for (int ks = 0; ks < DK; ++ks) {
+    const int ch = 32 * ks + 8 * g4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) qf[ks].u[e] = 0;
+    if (ch < a.d && rowok) {
+      const float* qp = a.q + (t * a.H + h) * a.d + ch;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qf[ks].h[e] = bf_bits(qp[e]);
+    }
+  }
+
+  const int p_first = past + row0, p_last = past + row0 + nrows - 1;
+  const bool win = a.window > 0;
+  const int lo_tile = win ? (p_first - a.window + 1 > 0 ? p_first - a.window + 1 : 0) : 0;
+  const int pl = lo_tile / PAGE, last = p_last / PAGE;
+  const int w_first = p_first + 16 * wave, w_last = (w_first + 15 < p_last ? w_first + 15 : p_last);
+  const int w_lo = win ? w_first - a.window + 1 : 0;
+  const bool wave_has_rows = 16 * wave < nrows;
+  const int my_lo = win ? qpos - a.window + 1 : 0;
+
+  const bf16* K = (const bf16*)a.kpages;
+  const bf16* V = (const bf16*)a.vpages;
+  const int* pages = bt.pages + (int64_t)b * bt.max_pages;
+
+  float m = -1e30f, l = 0.f;
+  f32x4 O[NEB];
+#pragma unroll
+  for (int eb = 0; eb < NEB; ++eb) O[eb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int pg = pl; pg <= last; ++pg) {
+    const int page = pages[pg];
+    const int k0 = pg * PAGE;
+    const bool wave_sees = wave_has_rows && k0 <= w_last && k0 + PAGE - 1 >= w_lo;
+    // ---- value tile -> LDS, transposed: lane = key, wavefront w takes channel groups w, w + 4, ... (16 bytes each)
+    __syncthreads();                                         // the previous page's tile has been read
+    const bf16* vsrc = V + (((int64_t)page * a.G + gk) * PAGE + lane) * a.ldv;
+#pragma unroll
+    for (int c0 = 0; c0 < NEB / 2; c0 += 4) {
+      Frag vreg[4];
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int e0 = 8 * (4 * (c0 + it) + wave);
+        if (e0 < a.vd) vreg[it].q = *reinterpret_cast<const uint4*>(vsrc + e0);
+      }
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int e0 = 8 * (4 * (c0 + it) + wave);
+        if (e0 < a.vd) {
+#pragma unroll
+          for (int u = 0; u < 8; ++u) vt[(e0 + u) * MF_LDV + lane] = vreg[it].h[u];
+        }
+      }
+    }
+    __syncthreads();
+    if (!wave_sees) continue;
+
+    // ---- S^T = K Q^T for the 4 key blocks of the page, K fragments from memory three 32-channel steps at a time
+    const bf16* kpage = K + (((int64_t)page * a.G + gk) * PAGE) * a.d;
+    f32x4 S[4];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) S[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks0 = 0; ks0 < DK; ks0 += 3) {
+      Frag kf[4][3];
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+          const int ch = 32 * (ks0 + j) + 8 * g4;
+          kf[kb][j].q = (ks0 + j < DK && ch < a.d) ? *reinterpret_cast<const uint4*>(kpage + (int64_t)(16 * kb + lq) * a.d + ch)
+                                                   : uint4{0, 0, 0, 0};
+        }
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+          if (ks0 + j < DK) S[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kb][j].v, qf[ks0 + j].v, S[kb], 0, 0, 0);
+    }
+    // ---- mask, online softmax (per-lane scalars of the lane's query), exponentials as two bfloat16 terms
+    Frag phi[2], plo[2];
+    const bool inner = k0 + PAGE - 1 <= w_first && (!win || k0 >= w_last - a.window + 1);
+    float mx = -1e30f;
+    if (inner) {
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          S[kb][i] *= a.scale;
+          mx = fmaxf(mx, S[kb][i]);
+        }
+    } else {
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = k0 + 16 * kb + 4 * g4 + i;
+          const bool vis = key <= qpos && key >= my_lo;
+          S[kb][i] = vis ? S[kb][i] * a.scale : -1e30f;
+          mx = fmaxf(mx, S[kb][i]);
+        }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mnew = fmaxf(m, mx);
+    const float corr = __expf(m - mnew);
+    float sum = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int i = 0; i < 4; i += 2) {
+        float p0 = S[kb][i] > -1e29f ? __expf(S[kb][i] - mnew) : 0.f;
+        float p1 = S[kb][i + 1] > -1e29f ? __expf(S[kb][i + 1] - mnew) : 0.f;
+        sum += p0 + p1;
+        const uint32_t h0 = __float_as_uint(p0) & 0xffff0000u, h1 = __float_as_uint(p1) & 0xffff0000u;
+        const uint32_t l0 = __float_as_uint(p0 - __uint_as_float(h0)), l1 = __float_as_uint(p1 - __uint_as_float(h1));
+        phi[kb >> 1].u[2 * (kb & 1) + (i >> 1)] = (h0 >> 16) | h1;
+        plo[kb >> 1].u[2 * (kb & 1) + (i >> 1)] = (l0 >> 16) | (l1 & 0xffff0000u);
+      }
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    l = l * corr + sum;
+    m = mnew;
+#pragma unroll
+    for (int eb = 0; eb < NEB; ++eb) O[eb] *= corr;
+    // ---- O^T += V^T P^T
+#pragma unroll
+    for (int eb = 0; eb < NEB; ++eb) {
+      if (eb < neb) {
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          Frag vf;
+          const uint16_t* vrow = vt + (16 * eb + lq) * MF_LDV + 32 * c + 4 * g4;
+          vf.d2[0] = *reinterpret_cast<const uint2*>(vrow);
+          vf.d2[1] = *reinterpret_cast<const uint2*>(vrow + 16);
+          O[eb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, phi[c].v, O[eb], 0, 0, 0);
+          O[eb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, plo[c].v, O[eb], 0, 0, 0);
+        }
+      }
+    }
+  }
+  if (!rowok) return;
+  if (a.sink) {
+    const float mnew = fmaxf(m, a.sink_score), corr = __expf(m - mnew);
+    l = l * corr + __expf(a.sink_score - mnew);
+#pragma unroll
+    for (int eb = 0; eb < NEB; ++eb) O[eb] *= corr;
+  }
+  const float f = a.out_scale / l;
+  uint16_t* orow = (uint16_t*)a.out + t * (int64_t)(a.H * a.vd) + (int64_t)h * a.vd;
+#pragma unroll
+  for (int eb = 0; eb < NEB; ++eb)
+    if (eb < neb) {
+      uint2 w;
+      w.x = (uint32_t)bf_bits(O[eb][0] * f) | ((uint32_t)bf_bits(O[eb][1] * f) << 16);
+      w.y = (uint32_t)bf_bits(O[eb][2] * f) | ((uint32_t)bf_bits(O[eb][3] * f) << 16);
+      *reinterpret_cast<uint2*>(orow + 16 * eb + 4 * g4) = w;
+    }
+}
+
+// 1 when the wide kernel serves this layout: one map, no kept first tokens, no output norm, no gate
+extern "C" int ragged_paged_attn_mfma_wide_ok(int d, int vd) {
+  return d % 8 == 0 && d <= 32 * 18 && vd % 16 == 0 && vd <= 16 * 32;
+}
+
+template <int DK, int NEB>
+static int launch_wide(AttnArgs a, Batch bt, unsigned grid, hipStream_t st) {
+  const size_t lds = (size_t)NEB * 16 * MF_LDV * sizeof(uint16_t);
+  static bool raised = false;                                 // tiles above 64 KB need the limit raised once per kernel
+  if (lds > 64 * 1024 && !raised) {
+    if (hipFuncSetAttribute((const void*)paged_attn_mfma_wide_kernel<DK, NEB>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess) return -3;
+    raised = true;
+  }
+  hipLaunchKernelGGL((paged_attn_mfma_wide_kernel<DK, NEB>), dim3(grid), dim3(256), lds, st, a, bt);
+  return 0;
+}
+
+extern "C" int ragged_paged_attn_mfma_wide(AttnArgs a, Batch bt, hipStream_t st) {
+  if (bt.T <= 0 || a.H <= 0 || a.G <= 0 || a.H % a.G || !ragged_paged_attn_mfma_wide_ok(a.d, a.vd)) return -1;
+  if (a.ldv < a.vd || a.ldv % 8 || a.keep_first > 0 || a.out_norm || a.gate) return -1;
+  if (!a.tiles || a.n_tiles <= 0 || (int64_t)a.n_tiles * a.H > 0x7fffffff) return -1;
+  const unsigned grid = (unsigned)(a.n_tiles * a.H);
+  const int dk = (a.d + 31) / 32, neb = a.vd / 16;
+  int rc;
+  if (dk <= 6 && neb <= 8) rc = launch_wide<6, 8>(a, bt, grid, st);
+  else if (dk <= 6 && neb <= 16) rc = launch_wide<6, 16>(a, bt, grid, st);
+  else if (dk <= 10 && neb <= 16) rc = launch_wide<10, 16>(a, bt, grid, st);
+  else if (dk <= 10) rc = launch_wide<10, 32>(a, bt, grid, st);
+  else rc = launch_wide<18, 32>(a, bt, grid, st);
+  if (rc) return rc;
+  return RAGGED_LAUNCH_OK();
+}
+
 // 1 when the MFMA kernel serves this head layout (bfloat16 only)
 extern "C" int ragged_paged_attn_mfma_ok(int d, int vd) {
   return d % 8 == 0 && d <= 32 * MF_DK && vd % 16 == 0 && vd <= 16 * MF_NEB;

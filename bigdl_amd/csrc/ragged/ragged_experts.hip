@@ -6,7 +6,7 @@
 
 using namespace ragged;
 
-constexpr int MOE_MAX_E = 256;      // experts
+constexpr int MOE_MAX_E = 512;      // experts
 constexpr int MOE_SLOTS = MOE_MAX_E / 64;
 
 // Scores s = softmax(W_r x) over all experts in float (x may be the bfloat16 rounding of the normed stream).  Experts
@@ -19,14 +19,41 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
                                                         int keep, int top, float scale) {
   __shared__ float z[MOE_MAX_E];
   __shared__ float gbest[64];
+  extern __shared__ __attribute__((aligned(16))) float xs[];       // the row as floats
   const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const T* xr = x + (int64_t)t * ldx;
-  for (int e = wave; e < E; e += 4) {
-    const float* w = wr + (int64_t)e * D;
-    float acc = 0.f;
-    for (int c = lane; c < D; c += 64) acc += w[c] * to_f(xr[c]);
-    acc = wave_sum(acc);
-    if (lane == 0) z[e] = acc;
+  for (int c = threadIdx.x; c < D; c += 256) xs[c] = to_f(xr[c]);
+  __syncthreads();
+  // two experts per wavefront and pass, 16 bytes of each router row per lane: eight loads in flight
+  const bool v4 = (D & 3) == 0;
+  for (int e0 = 2 * wave; e0 < E; e0 += 8) {
+    const int e1 = e0 + 1 < E ? e0 + 1 : e0;
+    const float* w0 = wr + (int64_t)e0 * D;
+    const float* w1 = wr + (int64_t)e1 * D;
+    float a0 = 0.f, a1 = 0.f;
+    if (v4) {
+      for (int c = 4 * lane; c < D; c += 1024) {
+        float4 p[4], q[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int cc = c + 256 * u < D ? c + 256 * u : c;
+          p[u] = *reinterpret_cast<const float4*>(w0 + cc);
+          q[u] = *reinterpret_cast<const float4*>(w1 + cc);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (c + 256 * u < D) {
+            const float4 xv = *reinterpret_cast<const float4*>(xs + c + 256 * u);
+            a0 += p[u].x * xv.x + p[u].y * xv.y + p[u].z * xv.z + p[u].w * xv.w;
+            a1 += q[u].x * xv.x + q[u].y * xv.y + q[u].z * xv.z + q[u].w * xv.w;
+          }
+      }
+    } else {
+      for (int c = lane; c < D; c += 64) { a0 += w0[c] * xs[c]; a1 += w1[c] * xs[c]; }
+    }
+    a0 = wave_sum(a0);
+    a1 = wave_sum(a1);
+    if (lane == 0) { z[e0] = a0; z[e1] = a1; }
   }
   __syncthreads();
   if (wave != 0) return;
@@ -95,9 +122,9 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
 
 extern "C" int ragged_moe_route(const void* x, int64_t ldx, const float* wr, int* idx, float* wts, int64_t rows, int D, int E,
                                 int groups, int keep, int top, float scale, int dtype, hipStream_t st) {
-  if (rows <= 0 || rows > 0x7fffffff || D <= 0 || E <= 0 || E > MOE_MAX_E || groups <= 0 || groups > 64 || E % groups) return -1;
+  if (rows <= 0 || rows > 0x7fffffff || D <= 0 || D > 12288 || E <= 0 || E > MOE_MAX_E || groups <= 0 || groups > 64 || E % groups) return -1;
   if (keep <= 0 || keep > groups || top <= 0 || top > keep * (E / groups)) return -1;
-  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((moe_route_kernel<T>), dim3((unsigned)rows), dim3(256), 0, st, (const T*)x, ldx, wr, idx,
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((moe_route_kernel<T>), dim3((unsigned)rows), dim3(256), D * sizeof(float), st, (const T*)x, ldx, wr, idx,
                                             wts, D, E, groups, keep, top, scale))
   return RAGGED_LAUNCH_OK();
 }

@@ -283,13 +283,15 @@ extern "C" int ragged_hgrn2_gates(const void* P, int64_t ldp, int q0, int f0, co
 constexpr int HG_DR = 32;
 constexpr int HG_SEG = HG_DR + 4;   // LDS floats per lane group and token (padding shifts the banks between groups)
 constexpr int HG_TBR = 64;          // TB * R <= this
+// pvd: value columns per head in P.  pvd = vd - 1: the state's last column takes a constant 1 as its value, so that it
+// carries n <- f n + g and the output's last column is n . q (the normaliser of an mLSTM head).
 // GIN: the input's weights come from a third array, S <- diag(f_t) S + g_t v_t^T (mLSTM hands in f = its decay
 // repeated over the rows and g = its input gate times the key); otherwise g = 1 - f.
 template <typename T, bool GIN>
 __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* __restrict__ qf, const float* __restrict__ ff,
                                                          const float* __restrict__ gf,
                                                          const T* __restrict__ P, int64_t ldp, int v0, float* __restrict__ state,
-                                                         float* __restrict__ out, int H, int d, int vd, int R, int TB, Batch bt) {
+                                                         float* __restrict__ out, int H, int d, int vd, int pvd, int R, int TB, Batch bt) {
   constexpr int NA = GIN ? 3 : 2;
   constexpr int HG_PRE = NA * HG_TBR * HG_DR / 256;
   extern __shared__ __attribute__((aligned(16))) float smem[];   // 2 x { q[TB][R][SEG], f[TB][R][SEG], (g,) v[TB][wcols] }
@@ -334,7 +336,7 @@ __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* __restrict
       float v = 0.f;
       if (e < TB * wcols) {
         const int tk = e / wcols, c = blockIdx.x * wcols + e % wcols;
-        if (i0 + tk < n && c < vd) v = to_f(P[(int64_t)(start + i0 + tk) * ldp + v0 + h * vd + c]);
+        if (i0 + tk < n && c < vd) v = c < pvd ? to_f(P[(int64_t)(start + i0 + tk) * ldp + v0 + h * pvd + c]) : 1.f;
       }
       prev[u] = v;
     }
@@ -403,8 +405,10 @@ __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* __restrict
 
 // gf null: the input's weight is 1 - f (HGRN2); otherwise the third gate array
 extern "C" int ragged_hgrn2_scan(const float* qf, const float* ff, const float* gf, const void* P, int64_t ldp, int v0,
-                                 float* state, float* out, int H, int d, int vd, Batch bt, int dtype, hipStream_t st) {
-  if (bt.B <= 0 || H <= 0 || d <= 0 || vd <= 0 || d > HG_DR * 64) return -1;
+                                 float* state, float* out, int H, int d, int vd, int ones_col, Batch bt, int dtype,
+                                 hipStream_t st) {
+  if (bt.B <= 0 || H <= 0 || d <= 0 || vd <= (ones_col ? 1 : 0) || d > HG_DR * 64) return -1;
+  const int pvd = ones_col ? vd - 1 : vd;
   int R = 1;
   while (R * HG_DR < d) R <<= 1;
   const int wcols = 4 * (64 / R);
@@ -415,9 +419,9 @@ extern "C" int ragged_hgrn2_scan(const float* qf, const float* ff, const float* 
   const dim3 grid((vd + wcols - 1) / wcols, H, bt.B);
   RAGGED_DISPATCH(dtype,
     if (gf) hipLaunchKernelGGL((hgrn2_scan_kernel<T, true>), grid, dim3(256), sm, st, qf, ff, gf, (const T*)P, ldp, v0, state, out,
-                               H, d, vd, R, TB, bt);
+                               H, d, vd, pvd, R, TB, bt);
     else hipLaunchKernelGGL((hgrn2_scan_kernel<T, false>), grid, dim3(256), sm, st, qf, ff, gf, (const T*)P, ldp, v0, state, out,
-                            H, d, vd, R, TB, bt))
+                            H, d, vd, pvd, R, TB, bt))
   return RAGGED_LAUNCH_OK();
 }
 

@@ -206,8 +206,8 @@ class RaggedDecoder:
             elif isinstance(m, Hgrn2):
                 s.append(("matrix", m.heads, m.dim, m.vdim))
             elif isinstance(m, Mlstm):
-                s.append(("matrix", m.heads, m.dim, m.vdim))
-                s.append(("vector", m.heads * (m.dim + 1)))     # per head: normaliser n[dim], then the running maximum
+                s.append(("matrix", m.heads, m.dim, m.vdim + 1))  # S and, as its last column, the normaliser n
+                s.append(("vector", m.heads))                   # the running maximum of every head
             specs[li] = s
         return specs
 
@@ -273,10 +273,12 @@ class RaggedDecoder:
         ops, pool = self.ops, self.pool
         hd, hv = m.heads * m.dim, m.heads * m.vdim
         # columns of P: q | k | v | output gate | input gates | forget gates
-        qf, ff, gf = ops.mlstm_prepare(P, 0, hd, 2 * hd + 2 * hv, lt.gate_bias, m.gate_cap, m.m_start, m.den_floor,
-                                       m.heads, m.dim, pool.vector[li], meta)
-        o = ops.hgrn2_scan(qf, ff, P, 2 * hd, pool.matrix[li], m.heads, m.dim, m.vdim, meta, gf=gf)
-        return ops.head_norm_gate(o, lt.o_norm, P, 2 * hd + hv, m.heads, m.vdim, self.cfg.norm_eps, self.act)
+        a, b, em = ops.mlstm_gates(P, 2 * hd + 2 * hv, lt.gate_bias, m.gate_cap, m.m_start, m.heads, pool.vector[li], meta)
+        qf, ff, gf = ops.mlstm_expand(P, 0, hd, a, b, m.heads, m.dim)
+        # the normaliser n rides along as one more column of the matrix memory (its value is the constant 1)
+        o = ops.hgrn2_scan(qf, ff, P, 2 * hd, pool.matrix[li], m.heads, m.dim, m.vdim + 1, meta, gf=gf, ones_col=True)
+        return ops.head_norm_gate(o, lt.o_norm, P, 2 * hd + hv, m.heads, m.vdim, self.cfg.norm_eps, self.act, em=em,
+                                  den_floor=m.den_floor)
 
     # rows per expert (on average) from which the experts run as dense products over their sorted rows; below, every
     # (row, chosen expert) pair is served by the row-wise kernels, which read no more than the chosen experts' weights

@@ -89,10 +89,11 @@ def lib():
         L.ragged_conv_state.argtypes = [vp, i64, ci, vp, ci, ci, _Batch, ci, vp]
         L.ragged_clamped_glu.argtypes = [vp, vp, i64, ci, cf, cf, ci, vp]
         L.ragged_hgrn2_gates.argtypes = [vp, i64, ci, ci, vp, vp, vp, vp, i64, ci, ci, vp]
-        L.ragged_hgrn2_scan.argtypes = [vp, vp, vp, vp, i64, ci, vp, vp, ci, ci, ci, _Batch, ci, vp]
+        L.ragged_hgrn2_scan.argtypes = [vp, vp, vp, vp, i64, ci, vp, vp, ci, ci, ci, ci, _Batch, ci, vp]
         L.ragged_post_norm_add.argtypes = [vp, vp, vp, vp, vp, i64, ci, cf, ci, vp]
-        L.ragged_mlstm_prepare.argtypes = [vp, i64, ci, ci, ci, vp, cf, cf, cf, vp, vp, vp, vp, ci, ci, _Batch, ci, vp]
-        L.ragged_head_norm_gate.argtypes = [vp, vp, vp, i64, ci, vp, i64, ci, ci, cf, ci, vp]
+        L.ragged_mlstm_gates.argtypes = [vp, i64, ci, vp, cf, cf, vp, vp, vp, vp, ci, _Batch, ci, vp]
+        L.ragged_mlstm_expand.argtypes = [vp, i64, ci, ci, vp, vp, vp, vp, vp, i64, ci, ci, ci, vp]
+        L.ragged_head_norm_gate.argtypes = [vp, vp, vp, i64, ci, vp, i64, ci, ci, cf, ci, vp, cf, ci, vp]
         L.ragged_moe_route.argtypes = [vp, i64, vp, vp, vp, i64, ci, ci, ci, ci, ci, cf, ci, vp]
         L.ragged_relu2.argtypes = [vp, vp, i64, ci, vp]
         L.ragged_moe_rows.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, i64, ci, ci, ci, ci, vp]
@@ -102,6 +103,8 @@ def lib():
         L.ragged_paged_attn.argtypes = [_AttnArgs, _Batch, ci, ci, vp]
         L.ragged_paged_attn_mfma.argtypes = [_AttnArgs, _Batch, ci, vp]
         L.ragged_paged_attn_mfma_ok.argtypes = [ci, ci]
+        L.ragged_paged_attn_mfma_wide.argtypes = [_AttnArgs, _Batch, vp]
+        L.ragged_paged_attn_mfma_wide_ok.argtypes = [ci, ci]
         _LIB = L
     return _LIB
 
@@ -255,6 +258,7 @@ class HipOps:
     def before_recording(self, meta):
         """Host-built tables a step needs (pinned allocations and copies cannot be recorded into a graph)."""
         meta.attn_split(self.mfma_min_rows)
+        meta.attn_split(1)
 
     def sum_group_norm(self, x, y, w, groups, alpha, eps, act, x_out=None, want_act=True):
         _f32(x, w, x_out)
@@ -338,11 +342,13 @@ class HipOps:
                                      ff.data_ptr(), rows, HD, _DT[P.dtype], _stream()), "hgrn2_gates")
         return qf, ff
 
-    def hgrn2_scan(self, qf, ff, P, v0, state, H, d, vd, meta, gf=None):
-        """S <- diag(f) S + g v^T, o = S^T q per head; g = 1 - f unless ``gf`` gives it."""
+    def hgrn2_scan(self, qf, ff, P, v0, state, H, d, vd, meta, gf=None, ones_col=False):
+        """S <- diag(f) S + g v^T, o = S^T q per head; g = 1 - f unless ``gf`` gives it.  ``ones_col``: the last of the
+        ``vd`` columns is not in P, its value is the constant 1 (state column n <- f n + g, output column n . q)."""
         _f32(qf, ff, state, gf)
         _act(P)
-        if qf.shape != (meta.T, H * d) or ff.shape != qf.shape or v0 + H * vd > P.shape[1] or P.shape[0] != meta.T \
+        oc = int(bool(ones_col))
+        if qf.shape != (meta.T, H * d) or ff.shape != qf.shape or v0 + H * (vd - oc) > P.shape[1] or P.shape[0] != meta.T \
                 or state.shape[1:] != (H, d, vd) or max(s[0] for s in meta.seqs) >= state.shape[0] \
                 or (gf is not None and gf.shape != qf.shape):
             raise ValueError("recurrent state / gates do not fit")
@@ -352,7 +358,7 @@ class HipOps:
         longest = max(n for _, _, n, _ in meta.seqs)
         if longest < 2 * self.scan_chunk:
             _ok(L.ragged_hgrn2_scan(qf.data_ptr(), ff.data_ptr(), g, P.data_ptr(), P.stride(0), v0, state.data_ptr(),
-                                    out.data_ptr(), H, d, vd, meta.c(), dt, st), "hgrn2_scan")
+                                    out.data_ptr(), H, d, vd, oc, meta.c(), dt, st), "hgrn2_scan")
             return out
         # long portions: chunks scanned side by side from zero, chunk-start states chained, chunks scanned again from them
         nc, cstart, zeros, ones, cid, cfirst, last = meta.chunks(self.scan_chunk)
@@ -363,13 +369,13 @@ class HipOps:
         def chunk_batch(past):
             return _Batch(None, None, cstart.data_ptr(), past.data_ptr(), cid.data_ptr(), None, meta.T, nc, 0)
         _ok(L.ragged_hgrn2_scan(qf.data_ptr(), ff.data_ptr(), g, P.data_ptr(), P.stride(0), v0, local.data_ptr(), out.data_ptr(),
-                                H, d, vd, chunk_batch(zeros), dt, st), "hgrn2_scan (chunks from zero)")
+                                H, d, vd, oc, chunk_batch(zeros), dt, st), "hgrn2_scan (chunks from zero)")
         _ok(L.ragged_hgrn2_chunk_decay(ff.data_ptr(), cstart.data_ptr(), decay.data_ptr(), nc, H * d, st), "hgrn2_chunk_decay")
         _ok(L.ragged_hgrn2_chunk_combine(state.data_ptr(), local.data_ptr(), decay.data_ptr(), begin.data_ptr(), cfirst.data_ptr(),
                                          meta.seq_past.data_ptr(), meta.seq_slot.data_ptr(), meta.B, H, d, vd, st),
             "hgrn2_chunk_combine")
         _ok(L.ragged_hgrn2_scan(qf.data_ptr(), ff.data_ptr(), g, P.data_ptr(), P.stride(0), v0, begin.data_ptr(), out.data_ptr(),
-                                H, d, vd, chunk_batch(ones), dt, st), "hgrn2_scan (chunks from their start states)")
+                                H, d, vd, oc, chunk_batch(ones), dt, st), "hgrn2_scan (chunks from their start states)")
         slots = torch.tensor([s[0] for s in meta.seqs], dtype=torch.int64, device=P.device)
         state[slots] = begin[torch.tensor(last, dtype=torch.int64, device=P.device)]     # every sequence's end state
         return out
@@ -408,6 +414,14 @@ class HipOps:
         a.ldv = vpages.shape[3]
         if sink is not None:
             a.sink, a.sink_score = 1, float(sink)
+        if kpages.dtype == torch.bfloat16 and self.mfma and maps == 1 and not lib().ragged_paged_attn_mfma_ok(d, vd) \
+                and lib().ragged_paged_attn_mfma_wide_ok(d, vd) and a.ldv % 8 == 0 and not keep_first and not out_norm \
+                and gate is None:
+            # rows too wide for the row-wise kernel's lanes: every portion and single token on the matrix cores
+            tiles, n_tiles, _, _ = meta.attn_split(1)
+            a.tiles, a.n_tiles = tiles.data_ptr(), n_tiles
+            _ok(lib().ragged_paged_attn_mfma_wide(a, meta.c(), _stream()), "paged_attn_mfma_wide")
+            return out
         if kpages.dtype == torch.bfloat16 and self.mfma and lib().ragged_paged_attn_mfma_ok(d, vd) and a.ldv % 8 == 0:
             # long portions on the matrix cores, single tokens and short portions row by row
             tiles, n_tiles, rows, n_rows = meta.attn_split(self.mfma_min_rows)
@@ -443,30 +457,47 @@ class HipOps:
             _ok(lib().ragged_relu2(A.data_ptr(), out.data_ptr(), A.numel(), _DT[A.dtype], _stream()), "relu2")
         return out
 
-    def head_norm_gate(self, o, w, P, g0, H, vd, eps, act):
-        _f32(o, w)
+    def head_norm_gate(self, o, w, P, g0, H, vd, eps, act, em=None, den_floor=0.0):
+        """each head's rows of ``o`` divided by their root mean square, times ``w``, times sigmoid(gate columns of P).  With
+        ``em`` [T, H]: ``o`` has vd + 1 columns per head and is first divided by max(|last column|, em) + den_floor."""
+        _f32(o, w, em)
         _act(P)
         T = o.shape[0]
-        if o.shape != (T, H * vd) or w.numel() != H * vd or P.shape[0] != T or g0 + H * vd > P.shape[1] or P.dtype != act:
+        ldo = vd + (0 if em is None else 1)
+        if o.shape != (T, H * ldo) or w.numel() != H * vd or P.shape[0] != T or g0 + H * vd > P.shape[1] or P.dtype != act \
+                or (em is not None and em.shape != (T, H)):
             raise ValueError("head outputs / gate columns do not fit")
         out = torch.empty(T, H * vd, dtype=act, device=o.device)
         _ok(lib().ragged_head_norm_gate(o.data_ptr(), w.data_ptr(), P.data_ptr(), P.stride(0), g0, out.data_ptr(), T, H, vd, eps,
-                                        _DT[act], _stream()), "head_norm_gate")
+                                        ldo, None if em is None else em.data_ptr(), den_floor, _DT[act], _stream()),
+            "head_norm_gate")
         return out
 
-    def mlstm_prepare(self, P, q0, k0, i0, gate_bias, cap, m_start, den_floor, H, d, vec, meta):
-        """The scalar part of the mLSTM recurrence over this step's rows; returns (q / denominator, decay, input gate
-        times key), each float [T, H d], for the matrix scan.  ``vec`` [slots, H (d + 1)] carries n and m."""
+    def mlstm_gates(self, P, i0, gate_bias, cap, m_start, H, mstate, meta):
+        """Soft-capped log gates of this step's rows (columns i0 .. of P: input gates, then forget gates) and the running
+        maximum m carried in ``mstate`` [slots, H]; returns the decay a, the input weight b and e^-m, float [T, H] each."""
         _act(P)
-        _f32(gate_bias, vec)
-        if P.shape[0] != meta.T or max(q0, k0) + H * d > P.shape[1] or i0 + 2 * H > P.shape[1] or gate_bias.numel() != 2 * H \
-                or vec.shape[1] != H * (d + 1) or max(s[0] for s in meta.seqs) >= vec.shape[0]:
+        _f32(gate_bias, mstate)
+        if P.shape[0] != meta.T or i0 + 2 * H > P.shape[1] or gate_bias.numel() != 2 * H or mstate.shape[1] != H \
+                or max(s[0] for s in meta.seqs) >= mstate.shape[0]:
             raise ValueError("gate columns / state slots do not fit")
-        qf = torch.empty(meta.T, H * d, dtype=torch.float32, device=P.device)
+        a = torch.empty(meta.T, H, dtype=torch.float32, device=P.device)
+        b, em = torch.empty_like(a), torch.empty_like(a)
+        _ok(lib().ragged_mlstm_gates(P.data_ptr(), P.stride(0), i0, gate_bias.data_ptr(), cap, m_start, mstate.data_ptr(),
+                                     a.data_ptr(), b.data_ptr(), em.data_ptr(), H, meta.c(), _DT[P.dtype], _stream()), "mlstm_gates")
+        return a, b, em
+
+    def mlstm_expand(self, P, q0, k0, a, b, H, d):
+        """The matrix scan's arrays: q dim^-1/2, the decay repeated over the rows, b k; float [T, H d] each."""
+        _act(P)
+        _f32(a, b)
+        T = P.shape[0]
+        if max(q0, k0) + H * d > P.shape[1] or a.shape != (T, H) or b.shape != (T, H):
+            raise ValueError("query / key columns do not fit")
+        qf = torch.empty(T, H * d, dtype=torch.float32, device=P.device)
         ff, gf = torch.empty_like(qf), torch.empty_like(qf)
-        _ok(lib().ragged_mlstm_prepare(P.data_ptr(), P.stride(0), q0, k0, i0, gate_bias.data_ptr(), cap, m_start, den_floor,
-                                       vec.data_ptr(), qf.data_ptr(), ff.data_ptr(), gf.data_ptr(), H, d, meta.c(), _DT[P.dtype],
-                                       _stream()), "mlstm_prepare")
+        _ok(lib().ragged_mlstm_expand(P.data_ptr(), P.stride(0), q0, k0, a.data_ptr(), b.data_ptr(), qf.data_ptr(), ff.data_ptr(),
+                                      gf.data_ptr(), T, H, d, _DT[P.dtype], _stream()), "mlstm_expand")
         return qf, ff, gf
 
     def moe_route(self, xa, w_router, groups, keep, top, scale):
@@ -583,14 +614,18 @@ class TorchOps:
         f = lower + (1 - lower) * torch.sigmoid(P[:, f0:f0 + HD].float() + fb)
         return q * torch.sigmoid(q), f
 
-    def hgrn2_scan(self, qf, ff, P, v0, state, H, d, vd, meta, gf=None):
+    def hgrn2_scan(self, qf, ff, P, v0, state, H, d, vd, meta, gf=None, ones_col=False):
         out = torch.empty(meta.T, H * vd, dtype=torch.float32, device=P.device)
+        pv = vd - int(bool(ones_col))
         for b, (slot, past, n, _) in enumerate(meta.seqs):
             S = state[slot].clone() if past > 0 else torch.zeros_like(state[slot])
             for i in range(n):
                 t = meta.start[b] + i
                 f = ff[t].view(H, d, 1)
-                S = f * S + (1 - f if gf is None else gf[t].view(H, d, 1)) * P[t, v0:v0 + H * vd].float().view(H, 1, vd)
+                v = P[t, v0:v0 + H * pv].float().view(H, 1, pv)
+                if ones_col:
+                    v = torch.cat([v, torch.ones(H, 1, 1)], -1)
+                S = f * S + (1 - f if gf is None else gf[t].view(H, d, 1)) * v
                 out[t] = (S * qf[t].view(H, d, 1)).sum(1).reshape(-1)
             state[slot] = S
         return out
@@ -645,32 +680,32 @@ class TorchOps:
     def relu2(self, A):
         return torch.relu(A.float()).pow(2).to(A.dtype)
 
-    def head_norm_gate(self, o, w, P, g0, H, vd, eps, act):
-        v = o.view(-1, H, vd)
+    def head_norm_gate(self, o, w, P, g0, H, vd, eps, act, em=None, den_floor=0.0):
+        v = o.view(o.shape[0], H, -1)
+        if em is not None:
+            v = v[..., :vd] / (torch.maximum(v[..., vd].abs(), em) + den_floor)[..., None]
         v = (v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)).reshape(-1, H * vd)
         return (v * w * torch.sigmoid(P[:, g0:g0 + H * vd].float())).to(act)
 
-    def mlstm_prepare(self, P, q0, k0, i0, gate_bias, cap, m_start, den_floor, H, d, vec, meta):
-        T = meta.T
-        q = P[:, q0:q0 + H * d].float().view(T, H, d) * d ** -0.5
-        k = P[:, k0:k0 + H * d].float().view(T, H, d)
-        gi = cap * torch.tanh((P[:, i0:i0 + H].float() + gate_bias[:H]) / cap)
-        gfo = F.logsigmoid(cap * torch.tanh((P[:, i0 + H:i0 + 2 * H].float() + gate_bias[H:]) / cap))
-        qf, ff, gf = torch.empty(T, H, d), torch.empty(T, H, d), torch.empty(T, H, d)
-        for b, (slot, past, n, _) in enumerate(meta.seqs):
-            st = vec[slot].view(H, d + 1)
-            nv = st[:, :d].clone() if past > 0 else torch.zeros(H, d)
-            m = st[:, d].clone() if past > 0 else torch.full((H,), float(m_start))
+    def mlstm_gates(self, P, i0, gate_bias, cap, m_start, H, mstate, meta):
+        li = cap * torch.tanh((P[:, i0:i0 + H].float() + gate_bias[:H]) / cap)
+        lf = F.logsigmoid(cap * torch.tanh((P[:, i0 + H:i0 + 2 * H].float() + gate_bias[H:]) / cap))
+        a, b, em = torch.empty_like(li), torch.empty_like(li), torch.empty_like(li)
+        for s, (slot, past, n, _) in enumerate(meta.seqs):
+            m = mstate[slot].clone() if past > 0 else torch.full((H,), float(m_start))
             for i in range(n):
-                t = meta.start[b] + i
-                m2 = torch.maximum(gfo[t] + m, gi[t])
-                a, bb = torch.exp(gfo[t] + m - m2), torch.exp(gi[t] - m2)
-                nv = a[:, None] * nv + bb[:, None] * k[t]
+                t = meta.start[s] + i
+                m2 = torch.maximum(lf[t] + m, li[t])
+                a[t], b[t], em[t] = torch.exp(lf[t] + m - m2), torch.exp(li[t] - m2), torch.exp(-m2)
                 m = m2
-                den = torch.maximum((nv * q[t]).sum(-1).abs(), torch.exp(-m)) + den_floor
-                qf[t], ff[t], gf[t] = q[t] / den[:, None], a[:, None].expand(H, d), bb[:, None] * k[t]
-            st[:, :d], st[:, d] = nv, m
-        return qf.view(T, -1), ff.reshape(T, -1), gf.view(T, -1)
+            mstate[slot] = m
+        return a, b, em
+
+    def mlstm_expand(self, P, q0, k0, a, b, H, d):
+        T = P.shape[0]
+        q = P[:, q0:q0 + H * d].float() * d ** -0.5
+        k = P[:, k0:k0 + H * d].float().view(T, H, d)
+        return q, a[:, :, None].expand(T, H, d).reshape(T, -1).contiguous(), (b[:, :, None] * k).reshape(T, -1)
 
     def moe_route(self, xa, w_router, groups, keep, top, scale):
         s = torch.softmax(xa.float() @ w_router.t(), -1)

@@ -318,7 +318,7 @@ def test_mlstm_recurrence_and_its_state(device, heads, dim, vdim, cap, portions)
          "o": torch.eye(H * e)}
     W = {k: v.double() for k, v in W.items()}
     ops = R.ops_for(device)
-    pool = PagedStatePool({0: [("matrix", H, d, e), ("vector", H * (d + 1))]}, 64 * 40, 1, torch.float32, device)
+    pool = PagedStatePool({0: [("matrix", H, d, e + 1), ("vector", H)]}, 64 * 40, 1, torch.float32, device)
     gate_bias = torch.cat([W["i.b"], W["f.b"]]).float().to(device)
     wcat = torch.cat([W["q"], W["k"], W["v"], W["g"], W["i"], W["f"]])
     for seq in range(2):
@@ -330,9 +330,11 @@ def test_mlstm_recurrence_and_its_state(device, heads, dim, vdim, cap, portions)
         for n in portions:
             meta = _meta_for(pool, slot, n, device)
             Pn = P[at:at + n].contiguous()
-            qf, ff, gf = ops.mlstm_prepare(Pn, 0, H * d, 2 * H * d + 2 * H * e, gate_bias, cap, 0.0, 1e-6, H, d, pool.vector[0], meta)
-            o = ops.hgrn2_scan(qf, ff, Pn, 2 * H * d, pool.matrix[0], H, d, e, meta, gf=gf)
-            out.append(ops.head_norm_gate(o, W["norm"].float().to(device), Pn, 2 * H * d + H * e, H, e, 1e-5, torch.float32))
+            a, b, em = ops.mlstm_gates(Pn, 2 * H * d + 2 * H * e, gate_bias, cap, 0.0, H, pool.vector[0], meta)
+            qf, ff, gf = ops.mlstm_expand(Pn, 0, H * d, a, b, H, d)
+            o = ops.hgrn2_scan(qf, ff, Pn, 2 * H * d, pool.matrix[0], H, d, e + 1, meta, gf=gf, ones_col=True)
+            out.append(ops.head_norm_gate(o, W["norm"].float().to(device), Pn, 2 * H * d + H * e, H, e, 1e-5, torch.float32,
+                                          em=em, den_floor=1e-6))
             pool.commit(slot, n)
             at += n
         close(torch.cat(out).double().cpu(), want, 2e-4)
@@ -479,7 +481,9 @@ def test_trace_runner_replays_steps(tmp_path):
 @pytest.mark.gpu
 @pytest.mark.parametrize("H,G,d,e,window,sink,shared", [(4, 2, 64, 128, 100, 0.0, False), (2, 2, 48, 96, 70, 1.5, False),
                                                        (3, 1, 16, 32, 0, -2.0, False), (4, 1, 80, 64, 66, None, True),
-                                                       (2, 1, 128, 112, 300, None, True)])
+                                                       (2, 1, 128, 112, 300, None, True), (4, 1, 144, 128, 66, None, True),
+                                                       (2, 1, 576, 512, 100, None, True), (2, 2, 200, 192, 0, 1.0, False),
+                                                       (3, 1, 328, 256, 130, None, True)])
 def test_matrix_core_attention_with_a_sink_and_with_values_inside_the_key_rows(H, G, d, e, window, sink, shared):
     """bfloat16 prompt portions (the MFMA kernel) and single tokens (the row-wise kernel) against the plain statement on
     the same bfloat16-rounded keys and values"""
@@ -494,7 +498,8 @@ def test_matrix_core_attention_with_a_sink_and_with_values_inside_the_key_rows(H
         js = [x for x in range(T) if O.visible(i, x, window)]
         for hh in range(H):
             gg = hh // (H // G)
-            qq = q[i, hh].bfloat16().double() if i < 190 else q[i, hh]          # the MFMA kernel rounds its queries
+            # the MFMA kernels round their queries; rows wider than 128 channels take them for single tokens too
+            qq = q[i, hh].bfloat16().double() if i < 190 or d > 128 else q[i, hh]
             want[i, hh] = (torch.softmax((k[js, gg] @ qq) * scale, 0) @ v[js, gg]) if sink is None else \
                 O.sink_attend(qq, k[js, gg], v[js, gg], scale, sink)
     got = _attend_through_pages("cuda", q, k, e if shared else v, [120, 70] + [1] * 10, window=window, scale=scale, sink=sink,
