@@ -284,8 +284,8 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_kernel(AttnArgs a, Batch 
 // attention has them after its queries are carried into the latent space (keys [latent row | rotated part], values the
 // latent row).  Same tile, same transposed scores, same softmax and same two-term weights as above; what differs is
 // where the operands live: the output tile alone takes up to 128 registers, so K fragments are not held a page ahead but
-// come from memory a few 32-channel steps at a time (the four wavefronts of a workgroup read the same page, so three of
-// four reads hit the CU's cache), and the value tile is brought in and transposed 128 channels at a time.
+// come from memory six 32-channel steps at a time (the four wavefronts of a workgroup read the same page, so three of
+// four reads hit the CU's cache), and the value tile's registers are requested one page ahead.
 template <int DK, int NEB>
 __global__ __launch_bounds__(256) void paged_attn_mfma_wide_kernel(AttnArgs a, Batch bt) {
   extern __shared__ __attribute__((aligned(16))) uint16_t vt[];                   // V^T [16 NEB][PAGE (+ pad)]
@@ -333,45 +333,50 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_wide_kernel(AttnArgs a, B
 #pragma unroll
   for (int eb = 0; eb < NEB; ++eb) O[eb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // this lane's share of a page's value tile (lane = key, wavefront w takes channel groups w, w + 4, ..., 16 bytes each),
+  // requested one page ahead so that it is in flight during the current page's arithmetic
+  Frag vreg[NEB / 2];
+  auto load_values = [&](int page) {
+    const bf16* vsrc = V + (((int64_t)page * a.G + gk) * PAGE + lane) * a.ldv;
+#pragma unroll
+    for (int it = 0; it < NEB / 2; ++it) {
+      const int e0 = 8 * (4 * it + wave);
+      if (e0 < a.vd) vreg[it].q = *reinterpret_cast<const uint4*>(vsrc + e0);
+    }
+  };
+  if (pl <= last) load_values(pages[pl]);
+
   for (int pg = pl; pg <= last; ++pg) {
     const int page = pages[pg];
     const int k0 = pg * PAGE;
     const bool wave_sees = wave_has_rows && k0 <= w_last && k0 + PAGE - 1 >= w_lo;
-    // ---- value tile -> LDS, transposed: lane = key, wavefront w takes channel groups w, w + 4, ... (16 bytes each)
+    // ---- value tile -> LDS, transposed
     __syncthreads();                                         // the previous page's tile has been read
-    const bf16* vsrc = V + (((int64_t)page * a.G + gk) * PAGE + lane) * a.ldv;
 #pragma unroll
-    for (int c0 = 0; c0 < NEB / 2; c0 += 4) {
-      Frag vreg[4];
+    for (int it = 0; it < NEB / 2; ++it) {
+      const int e0 = 8 * (4 * it + wave);
+      if (e0 < a.vd) {
 #pragma unroll
-      for (int it = 0; it < 4; ++it) {
-        const int e0 = 8 * (4 * (c0 + it) + wave);
-        if (e0 < a.vd) vreg[it].q = *reinterpret_cast<const uint4*>(vsrc + e0);
-      }
-#pragma unroll
-      for (int it = 0; it < 4; ++it) {
-        const int e0 = 8 * (4 * (c0 + it) + wave);
-        if (e0 < a.vd) {
-#pragma unroll
-          for (int u = 0; u < 8; ++u) vt[(e0 + u) * MF_LDV + lane] = vreg[it].h[u];
-        }
+        for (int u = 0; u < 8; ++u) vt[(e0 + u) * MF_LDV + lane] = vreg[it].h[u];
       }
     }
     __syncthreads();
+    if (pg < last) load_values(pages[pg + 1]);
     if (!wave_sees) continue;
 
-    // ---- S^T = K Q^T for the 4 key blocks of the page, K fragments from memory three 32-channel steps at a time
+    // ---- S^T = K Q^T for the 4 key blocks of the page, K fragments from memory KS 32-channel steps at a time
     const bf16* kpage = K + (((int64_t)page * a.G + gk) * PAGE) * a.d;
     f32x4 S[4];
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) S[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    constexpr int KS = DK % 6 == 0 ? 6 : 5;
 #pragma unroll
-    for (int ks0 = 0; ks0 < DK; ks0 += 3) {
-      Frag kf[4][3];
+    for (int ks0 = 0; ks0 < DK; ks0 += KS) {
+      Frag kf[4][KS];
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-        for (int j = 0; j < 3; ++j) {
+        for (int j = 0; j < KS; ++j) {
           const int ch = 32 * (ks0 + j) + 8 * g4;
           kf[kb][j].q = (ks0 + j < DK && ch < a.d) ? *reinterpret_cast<const uint4*>(kpage + (int64_t)(16 * kb + lq) * a.d + ch)
                                                    : uint4{0, 0, 0, 0};
@@ -379,7 +384,7 @@ __global__ __launch_bounds__(256) void paged_attn_mfma_wide_kernel(AttnArgs a, B
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-        for (int j = 0; j < 3; ++j)
+        for (int j = 0; j < KS; ++j)
           if (ks0 + j < DK) S[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kb][j].v, qf[ks0 + j].v, S[kb], 0, 0, 0);
     }
     // ---- mask, online softmax (per-lane scalars of the lane's query), exponentials as two bfloat16 terms

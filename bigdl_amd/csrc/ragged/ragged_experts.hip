@@ -266,3 +266,25 @@ extern "C" int ragged_moe_rows(const void* x, int64_t ldx, const int* idx, const
                        (const T*)A, idx, wts, (const T*)w_dn, (const T*)base, (T*)y, D, ff, top, vd))
   return RAGGED_LAUNCH_OK();
 }
+
+// y[t, :] = base[t, :] + sum_j wts[t, j] * ys[place[t, j], :]: the experts' outputs, computed on rows sorted by expert,
+// brought back to their rows (every row sums its own terms in the order of its choices).
+template <typename T>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const T* __restrict__ ys, const int* __restrict__ place,
+                                                          const float* __restrict__ wts, const T* __restrict__ base,
+                                                          T* __restrict__ y, int D, int top) {
+  const int64_t t = blockIdx.x;
+  for (int c = threadIdx.x; c < D; c += 256) {
+    float acc = base ? to_f(base[t * D + c]) : 0.f;
+    for (int j = 0; j < top; ++j) acc += wts[t * top + j] * to_f(ys[(int64_t)place[t * top + j] * D + c]);
+    y[t * D + c] = from_f<T>(acc);
+  }
+}
+
+extern "C" int ragged_moe_combine(const void* ys, const int* place, const float* wts, const void* base, void* y, int64_t rows, int D,
+                                  int top, int dtype, hipStream_t st) {
+  if (rows <= 0 || rows > 0x7fffffff || D <= 0 || top <= 0) return -1;
+  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((moe_combine_kernel<T>), dim3((unsigned)rows), dim3(256), 0, st, (const T*)ys, place, wts,
+                                            (const T*)base, (T*)y, D, top))
+  return RAGGED_LAUNCH_OK();
+}

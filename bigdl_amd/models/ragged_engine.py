@@ -292,19 +292,28 @@ class RaggedDecoder:
             base = F.linear(ops.relu2(F.linear(xa, lt.w_sup)), lt.w_sdn)
         if meta.T * f.top < self.moe_dense_rows * f.experts:
             return ops.moe_rows(xa, idx, wts, lt.w_up, lt.w_dn, base)
-        y = torch.zeros(meta.T, self.cfg.width, dtype=torch.float32, device=self.device) if base is None else base.float()
+        # rows sorted by expert: one gather, two library products per expert on its run of rows, one weighted sum per row
+        T, top = meta.T, f.top
         order = idx.view(-1).sort(stable=True)
-        counts = torch.bincount(order.values, minlength=f.experts).tolist()     # (the host learns the segment sizes)
-        pair = order.indices
-        rows, wsel = pair // f.top, wts.view(-1)[pair]
+        counts = torch.bincount(order.values, minlength=f.experts).tolist()     # (the host learns the runs' lengths)
+        pair = order.indices                                                    # pair t * top + j at every sorted place
+        xs = xa[pair // top]
+        A = torch.empty(T * top, f.ff, dtype=self.act, device=self.device)
         at = 0
         for e, c in enumerate(counts):
             if c:
-                r = rows[at:at + c]
-                out = F.linear(ops.relu2(F.linear(xa[r], lt.w_up[e])), lt.w_dn[e])
-                y.index_add_(0, r, out.float() * wsel[at:at + c, None])
+                torch.mm(xs[at:at + c], lt.w_up[e].t(), out=A[at:at + c])
                 at += c
-        return y.to(self.act)
+        A = ops.relu2(A)
+        ys = torch.empty(T * top, self.cfg.width, dtype=self.act, device=self.device)
+        at = 0
+        for e, c in enumerate(counts):
+            if c:
+                torch.mm(A[at:at + c], lt.w_dn[e].t(), out=ys[at:at + c])
+                at += c
+        place = torch.empty_like(pair)
+        place[pair] = torch.arange(T * top, device=self.device)
+        return ops.moe_combine(ys, place.view(T, top).to(torch.int32), wts, base)
 
     def _hgrn2(self, li, m: Hgrn2, lt: LayerTensors, P, meta):
         ops = self.ops

@@ -96,6 +96,7 @@ def lib():
         L.ragged_head_norm_gate.argtypes = [vp, vp, vp, i64, ci, vp, i64, ci, ci, cf, ci, vp, cf, ci, vp]
         L.ragged_moe_route.argtypes = [vp, i64, vp, vp, vp, i64, ci, ci, ci, ci, ci, cf, ci, vp]
         L.ragged_relu2.argtypes = [vp, vp, i64, ci, vp]
+        L.ragged_moe_combine.argtypes = [vp, vp, vp, vp, vp, i64, ci, ci, ci, vp]
         L.ragged_moe_rows.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, i64, ci, ci, ci, ci, vp]
         L.ragged_hgrn2_chunk_decay.argtypes = [vp, vp, vp, ci, ci, vp]
         L.ragged_hgrn2_chunk_combine.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, vp]
@@ -513,6 +514,21 @@ class HipOps:
                                    keep, top, scale, _DT[xa.dtype], _stream()), "moe_route")
         return idx, wts
 
+    def moe_combine(self, ys, place, wts, base):
+        """y[t] = base[t] + sum_j wts[t, j] * ys[place[t, j]]"""
+        _act(ys, base)
+        _f32(wts)
+        T, top = place.shape
+        D = ys.shape[1]
+        if ys.shape[0] != T * top or not ys.is_contiguous() or place.dtype != torch.int32 or not place.is_contiguous() \
+                or wts.shape != (T, top) or (base is not None and (base.shape != (T, D) or base.dtype != ys.dtype
+                                                                   or not base.is_contiguous())):
+            raise ValueError("expert outputs / places do not fit")
+        y = torch.empty(T, D, dtype=ys.dtype, device=ys.device)
+        _ok(lib().ragged_moe_combine(ys.data_ptr(), place.data_ptr(), wts.data_ptr(), None if base is None else base.data_ptr(),
+                                     y.data_ptr(), T, D, top, _DT[ys.dtype], _stream()), "moe_combine")
+        return y
+
     def moe_rows(self, xa, idx, wts, w_up, w_dn, base):
         """y = base + sum over a row's chosen experts of weight * W_down relu(W_up x)^2, every pair served on its own."""
         _act(xa, w_up, w_dn, base)
@@ -715,6 +731,12 @@ class TorchOps:
         kept.scatter_(1, best.topk(keep, -1).indices, True)
         idx = s.masked_fill(~kept.repeat_interleave(E // groups, 1), -1.0).topk(top, -1).indices
         return idx.to(torch.int32), s.gather(1, idx) * scale
+
+    def moe_combine(self, ys, place, wts, base):
+        y = torch.zeros(place.shape[0], ys.shape[1]) if base is None else base.float().clone()
+        for j in range(place.shape[1]):
+            y += wts[:, j, None] * ys[place[:, j].long()].float()
+        return y.to(ys.dtype)
 
     def moe_rows(self, xa, idx, wts, w_up, w_dn, base):
         y = torch.zeros(xa.shape[0], w_dn.shape[1]) if base is None else base.float().clone()
