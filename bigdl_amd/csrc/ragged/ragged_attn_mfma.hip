@@ -502,6 +502,204 @@ extern "C" int ragged_paged_attn_mfma_wide(AttnArgs a, Batch bt, hipStream_t st)
   return RAGGED_LAUNCH_OK();
 }
 
+// Wide rows, single tokens and short portions: one workgroup serves one token row and 16 query heads that share a
+// key/value head -- the heads are the 16 columns of the score tile, so a page's keys are read once for all of them.
+// The four wavefronts split a page's keys for the scores (wavefront w: keys 16 w .. 16 w + 15, K fragments straight from
+// memory, requested one page ahead) and the value channels for the weighted sum (wavefront w: a quarter of the 16-channel
+// blocks); in between, the page's maxima, sums and exponentials (two bfloat16 terms each, already in the layout of the
+// second product's operand) cross the wavefronts through LDS.
+template <int DK, int NEB>
+__global__ __launch_bounds__(256) void paged_attn_mfma_heads_kernel(AttnArgs a, Batch bt) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t vt[];                   // V^T [16 NEB][PAGE (+ pad)]
+  uint4* pbuf = reinterpret_cast<uint4*>(vt + NEB * 16 * MF_LDV);                 // [4 key blocks][64 lanes]
+  float* smax = reinterpret_cast<float*>(pbuf + 256);                             // [4][16]
+  float* ssum = smax + 64;                                                        // [4][16]
+  constexpr int NE = NEB / 4;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int lq = lane & 15, g4 = lane >> 4;
+  const int share = a.H / a.G, nblk = (share + 15) / 16;
+  const int item = blockIdx.x, ri = item / (a.G * nblk), rem = item % (a.G * nblk);
+  const int gk = rem / nblk, blk = rem % nblk;
+  const int64_t t = a.rows ? a.rows[ri] : ri;
+  const int b = bt.tok_seq[t], qpos = bt.tok_pos[t];
+  const bool headok = blk * 16 + lq < share;
+  const int h = gk * share + (headok ? blk * 16 + lq : 0);
+  const int neb = a.vd / 16;
+
+  Frag qf[DK];
+#pragma unroll
+  for (int ks = 0; ks < DK; ++ks) {
+    const int ch = 32 * ks + 8 * g4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) qf[ks].u[e] = 0;
+    if (ch < a.d && headok) {
+      const float* qp = a.q + (t * a.H + h) * a.d + ch;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qf[ks].h[e] = bf_bits(qp[e]);
+    }
+  }
+  const bool win = a.window > 0;
+  const int lo = win ? (qpos - a.window + 1 > 0 ? qpos - a.window + 1 : 0) : 0;
+  const int pl = lo / PAGE, last = qpos / PAGE;
+  const bf16* K = (const bf16*)a.kpages;
+  const bf16* V = (const bf16*)a.vpages;
+  const int* pages = bt.pages + (int64_t)b * bt.max_pages;
+
+  float m = -1e30f, l = 0.f;
+  f32x4 O[NE];
+#pragma unroll
+  for (int e = 0; e < NE; ++e) O[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  Frag vreg[NEB / 2], kfn[DK];
+  auto load_page = [&](int page) {
+    const bf16* vsrc = V + (((int64_t)page * a.G + gk) * PAGE + lane) * a.ldv;
+#pragma unroll
+    for (int it = 0; it < NEB / 2; ++it) {
+      const int e0 = 8 * (4 * it + wave);
+      if (e0 < a.vd) vreg[it].q = *reinterpret_cast<const uint4*>(vsrc + e0);
+    }
+    const bf16* krow = K + (((int64_t)page * a.G + gk) * PAGE + 16 * wave + lq) * a.d;
+#pragma unroll
+    for (int ks = 0; ks < DK; ++ks) {
+      const int ch = 32 * ks + 8 * g4;
+      kfn[ks].q = ch < a.d ? *reinterpret_cast<const uint4*>(krow + ch) : uint4{0, 0, 0, 0};
+    }
+  };
+  load_page(pages[pl]);
+
+  for (int pg = pl; pg <= last; ++pg) {
+    const int k0 = pg * PAGE;
+    Frag kf[DK];
+#pragma unroll
+    for (int ks = 0; ks < DK; ++ks) kf[ks].q = kfn[ks].q;
+    __syncthreads();                                         // the previous page's tile and exponentials have been read
+#pragma unroll
+    for (int it = 0; it < NEB / 2; ++it) {
+      const int e0 = 8 * (4 * it + wave);
+      if (e0 < a.vd) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) vt[(e0 + u) * MF_LDV + lane] = vreg[it].h[u];
+      }
+    }
+    if (pg < last) load_page(pages[pg + 1]);
+    // ---- scores of this wavefront's 16 keys against the 16 heads
+    f32x4 S = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < DK; ++ks) S = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks].v, qf[ks].v, S, 0, 0, 0);
+    float mx = -1e30f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = k0 + 16 * wave + 4 * g4 + i;
+      S[i] = (key <= qpos && key >= lo) ? S[i] * a.scale : -1e30f;
+      mx = fmaxf(mx, S[i]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    if (g4 == 0) smax[wave * 16 + lq] = mx;
+    __syncthreads();
+    const float pm = fmaxf(fmaxf(smax[lq], smax[16 + lq]), fmaxf(smax[32 + lq], smax[48 + lq]));
+    const float mnew = fmaxf(m, pm);
+    const float corr = __expf(m - mnew);
+    float p[4], sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      p[i] = S[i] > -1e29f ? __expf(S[i] - mnew) : 0.f;
+      sum += p[i];
+    }
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    if (g4 == 0) ssum[wave * 16 + lq] = sum;
+    {
+      uint32_t hi[4], lw[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        hi[i] = __float_as_uint(p[i]) & 0xffff0000u;
+        lw[i] = __float_as_uint(p[i] - __uint_as_float(hi[i]));
+      }
+      pbuf[wave * 64 + lane] = uint4{(hi[0] >> 16) | hi[1], (hi[2] >> 16) | hi[3], (lw[0] >> 16) | (lw[1] & 0xffff0000u),
+                                     (lw[2] >> 16) | (lw[3] & 0xffff0000u)};
+    }
+    __syncthreads();
+    l = l * corr + ((ssum[lq] + ssum[16 + lq]) + (ssum[32 + lq] + ssum[48 + lq]));
+    m = mnew;
+    Frag phi[2], plo[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const uint4 x0 = pbuf[(2 * c) * 64 + lane], x1 = pbuf[(2 * c + 1) * 64 + lane];
+      phi[c].u[0] = x0.x; phi[c].u[1] = x0.y; phi[c].u[2] = x1.x; phi[c].u[3] = x1.y;
+      plo[c].u[0] = x0.z; plo[c].u[1] = x0.w; plo[c].u[2] = x1.z; plo[c].u[3] = x1.w;
+    }
+    // ---- this wavefront's value channels
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+      const int eb = wave * NE + e;
+      O[e] *= corr;
+      if (eb < neb) {
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          Frag vf;
+          const uint16_t* vrow = vt + (16 * eb + lq) * MF_LDV + 32 * c + 4 * g4;
+          vf.d2[0] = *reinterpret_cast<const uint2*>(vrow);
+          vf.d2[1] = *reinterpret_cast<const uint2*>(vrow + 16);
+          O[e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, phi[c].v, O[e], 0, 0, 0);
+          O[e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, plo[c].v, O[e], 0, 0, 0);
+        }
+      }
+    }
+  }
+  if (!headok) return;
+  float corr = 1.0f;
+  if (a.sink) {
+    const float mnew = fmaxf(m, a.sink_score);
+    corr = __expf(m - mnew);
+    l = l * corr + __expf(a.sink_score - mnew);
+  }
+  const float f = a.out_scale * corr / l;
+  uint16_t* orow = (uint16_t*)a.out + t * (int64_t)(a.H * a.vd) + (int64_t)h * a.vd;
+#pragma unroll
+  for (int e = 0; e < NE; ++e) {
+    const int eb = wave * NE + e;
+    if (eb < neb) {
+      uint2 w;
+      w.x = (uint32_t)bf_bits(O[e][0] * f) | ((uint32_t)bf_bits(O[e][1] * f) << 16);
+      w.y = (uint32_t)bf_bits(O[e][2] * f) | ((uint32_t)bf_bits(O[e][3] * f) << 16);
+      *reinterpret_cast<uint2*>(orow + 16 * eb + 4 * g4) = w;
+    }
+  }
+}
+
+template <int DK, int NEB>
+static int launch_heads(AttnArgs a, Batch bt, unsigned grid, hipStream_t st) {
+  const size_t lds = (size_t)NEB * 16 * MF_LDV * sizeof(uint16_t) + 256 * sizeof(uint4) + 128 * sizeof(float);
+  static bool raised = false;
+  if (lds > 64 * 1024 && !raised) {
+    if (hipFuncSetAttribute((const void*)paged_attn_mfma_heads_kernel<DK, NEB>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess) return -3;
+    raised = true;
+  }
+  hipLaunchKernelGGL((paged_attn_mfma_heads_kernel<DK, NEB>), dim3(grid), dim3(256), lds, st, a, bt);
+  return 0;
+}
+
+// token rows a.rows[0 .. n_rows) (all T rows without a list)
+extern "C" int ragged_paged_attn_mfma_heads(AttnArgs a, Batch bt, hipStream_t st) {
+  if (bt.T <= 0 || a.H <= 0 || a.G <= 0 || a.H % a.G || !ragged_paged_attn_mfma_wide_ok(a.d, a.vd)) return -1;
+  if (a.ldv < a.vd || a.ldv % 8 || a.keep_first > 0 || a.out_norm || a.gate) return -1;
+  const int nrows = a.rows ? a.n_rows : bt.T;
+  const int nblk = (a.H / a.G + 15) / 16;
+  if (nrows <= 0 || (int64_t)nrows * a.G * nblk > 0x7fffffff) return -1;
+  const unsigned grid = (unsigned)(nrows * a.G * nblk);
+  const int dk = (a.d + 31) / 32, neb = a.vd / 16;
+  int rc;
+  if (dk <= 6 && neb <= 8) rc = launch_heads<6, 8>(a, bt, grid, st);
+  else if (dk <= 6 && neb <= 16) rc = launch_heads<6, 16>(a, bt, grid, st);
+  else if (dk <= 10 && neb <= 16) rc = launch_heads<10, 16>(a, bt, grid, st);
+  else if (dk <= 10) rc = launch_heads<10, 32>(a, bt, grid, st);
+  else rc = launch_heads<18, 32>(a, bt, grid, st);
+  if (rc) return rc;
+  return RAGGED_LAUNCH_OK();
+}
+
 // 1 when the MFMA kernel serves this head layout (bfloat16 only)
 extern "C" int ragged_paged_attn_mfma_ok(int d, int vd) {
   return d % 8 == 0 && d <= 32 * MF_DK && vd % 16 == 0 && vd <= 16 * MF_NEB;

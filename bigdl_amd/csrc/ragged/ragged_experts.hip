@@ -149,8 +149,7 @@ extern "C" int ragged_relu2(const void* a, void* out, int64_t n, int dtype, hipS
 template <typename T> struct WVec;
 template <> struct WVec<bf16> {
   static constexpr int N = 8;
-  static __device__ __forceinline__ void load(const bf16* p, float* o) {
-    const uint4 u = *reinterpret_cast<const uint4*>(p);
+  static __device__ __forceinline__ void unpack(const uint4& u, float* o) {
     const uint32_t w[4] = {u.x, u.y, u.z, u.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -161,9 +160,8 @@ template <> struct WVec<bf16> {
 };
 template <> struct WVec<float> {
   static constexpr int N = 4;
-  static __device__ __forceinline__ void load(const float* p, float* o) {
-    const float4 u = *reinterpret_cast<const float4*>(p);
-    o[0] = u.x; o[1] = u.y; o[2] = u.z; o[3] = u.w;
+  static __device__ __forceinline__ void unpack(const uint4& u, float* o) {
+    o[0] = __uint_as_float(u.x); o[1] = __uint_as_float(u.y); o[2] = __uint_as_float(u.z); o[3] = __uint_as_float(u.w);
   }
 };
 
@@ -176,14 +174,30 @@ __device__ __forceinline__ void rows_dot(const T* __restrict__ w, int64_t K, int
 #pragma unroll
   for (int r = 0; r < R; ++r) acc[r] = 0.f;
   if (vec) {
-    for (int c = lane * N; c < K; c += 64 * N) {
-      float wv[R][N];
+    // four strides of every row requested before the first is used: 4 R loads of 16 bytes in flight per lane
+    constexpr int UN = 4;
+    for (int c0 = lane * N; c0 < K; c0 += UN * 64 * N) {
+      uint4 raw[UN][R];
 #pragma unroll
-      for (int r = 0; r < R; ++r) WVec<T>::load(w + (int64_t)(r < nrows ? r : nrows - 1) * K + c, wv[r]);
+      for (int u = 0; u < UN; ++u) {
+        const int c = c0 + u * 64 * N < K ? c0 + u * 64 * N : c0;
 #pragma unroll
-      for (int r = 0; r < R; ++r)
+        for (int r = 0; r < R; ++r)
+          raw[u][r] = *reinterpret_cast<const uint4*>(w + (int64_t)(r < nrows ? r : nrows - 1) * K + c);
+      }
 #pragma unroll
-        for (int e = 0; e < N; ++e) acc[r] += wv[r][e] * xs[c + e];
+      for (int u = 0; u < UN; ++u) {
+        const int c = c0 + u * 64 * N;
+        if (c < K) {
+#pragma unroll
+          for (int r = 0; r < R; ++r) {
+            float wv[N];
+            WVec<T>::unpack(raw[u][r], wv);
+#pragma unroll
+            for (int e = 0; e < N; ++e) acc[r] += wv[e] * xs[c + e];
+          }
+        }
+      }
     }
   } else {
     for (int c = lane; c < K; c += 64)

@@ -53,12 +53,45 @@ __device__ __forceinline__ float block_sum_256(float v, float* red) {
   return (red[0] + red[1]) + (red[2] + red[3]);
 }
 
-template <typename T>
+// NV > 0: rows of at most 256 NV channels, each thread keeps its NV sums in registers (every operand is read once);
+// NV = 0: any width, the passes re-read what they need.
+template <typename T, int NV>
 __global__ __launch_bounds__(256) void post_norm_add_kernel(float* __restrict__ x, const T* __restrict__ y,
                                                             const float* __restrict__ w_post, const float* __restrict__ w_next,
                                                             T* __restrict__ xa, int D, float eps) {
   __shared__ float red[8];
   const int64_t base = (int64_t)blockIdx.x * D;
+  if (NV > 0) {
+    float yv[NV > 0 ? NV : 1], xv[NV > 0 ? NV : 1], wp[NV > 0 ? NV : 1], wn[NV > 0 ? NV : 1];
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int c = threadIdx.x + 256 * u;
+      const bool ok = c < D;
+      yv[u] = ok ? to_f(y[base + c]) : 0.f;
+      xv[u] = ok ? x[base + c] : 0.f;
+      wp[u] = ok ? w_post[c] : 0.f;
+      wn[u] = (ok && xa) ? w_next[c] : 0.f;
+      ss += yv[u] * yv[u];
+    }
+    const float r1 = 1.0f / sqrtf(block_sum_256(ss, red) / (float)D + eps);
+    ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int c = threadIdx.x + 256 * u;
+      xv[u] += yv[u] * r1 * wp[u];
+      if (c < D) x[base + c] = xv[u];
+      ss += xv[u] * xv[u];
+    }
+    if (!xa) return;
+    const float r2 = 1.0f / sqrtf(block_sum_256(ss, red + 4) / (float)D + eps);
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int c = threadIdx.x + 256 * u;
+      if (c < D) xa[base + c] = from_f<T>(xv[u] * r2 * wn[u]);
+    }
+    return;
+  }
   float ss = 0.f;
   for (int c = threadIdx.x; c < D; c += 256) { const float v = to_f(y[base + c]); ss += v * v; }
   const float r1 = 1.0f / sqrtf(block_sum_256(ss, red) / (float)D + eps);
@@ -76,8 +109,13 @@ __global__ __launch_bounds__(256) void post_norm_add_kernel(float* __restrict__ 
 extern "C" int ragged_post_norm_add(float* x, const void* y, const float* w_post, const float* w_next, void* xa, int64_t rows,
                                     int D, float eps, int dtype, hipStream_t st) {
   if (rows <= 0 || D <= 0 || rows > 0x7fffffff || !x || !y || !w_post || (xa && !w_next)) return -1;
-  RAGGED_DISPATCH(dtype, hipLaunchKernelGGL((post_norm_add_kernel<T>), dim3((unsigned)rows), dim3(256), 0, st, x, (const T*)y,
-                                            w_post, w_next, (T*)xa, D, eps))
+  RAGGED_DISPATCH(dtype,
+    if (D <= 1024) hipLaunchKernelGGL((post_norm_add_kernel<T, 4>), dim3((unsigned)rows), dim3(256), 0, st, x, (const T*)y, w_post,
+                                      w_next, (T*)xa, D, eps);
+    else if (D <= 4096) hipLaunchKernelGGL((post_norm_add_kernel<T, 16>), dim3((unsigned)rows), dim3(256), 0, st, x, (const T*)y,
+                                           w_post, w_next, (T*)xa, D, eps);
+    else hipLaunchKernelGGL((post_norm_add_kernel<T, 0>), dim3((unsigned)rows), dim3(256), 0, st, x, (const T*)y, w_post, w_next,
+                            (T*)xa, D, eps))
   return RAGGED_LAUNCH_OK();
 }
 

@@ -105,6 +105,7 @@ def lib():
         L.ragged_paged_attn_mfma.argtypes = [_AttnArgs, _Batch, ci, vp]
         L.ragged_paged_attn_mfma_ok.argtypes = [ci, ci]
         L.ragged_paged_attn_mfma_wide.argtypes = [_AttnArgs, _Batch, vp]
+        L.ragged_paged_attn_mfma_heads.argtypes = [_AttnArgs, _Batch, vp]
         L.ragged_paged_attn_mfma_wide_ok.argtypes = [ci, ci]
         _LIB = L
     return _LIB
@@ -259,7 +260,6 @@ class HipOps:
     def before_recording(self, meta):
         """Host-built tables a step needs (pinned allocations and copies cannot be recorded into a graph)."""
         meta.attn_split(self.mfma_min_rows)
-        meta.attn_split(1)
 
     def sum_group_norm(self, x, y, w, groups, alpha, eps, act, x_out=None, want_act=True):
         _f32(x, w, x_out)
@@ -418,10 +418,15 @@ class HipOps:
         if kpages.dtype == torch.bfloat16 and self.mfma and maps == 1 and not lib().ragged_paged_attn_mfma_ok(d, vd) \
                 and lib().ragged_paged_attn_mfma_wide_ok(d, vd) and a.ldv % 8 == 0 and not keep_first and not out_norm \
                 and gate is None:
-            # rows too wide for the row-wise kernel's lanes: every portion and single token on the matrix cores
-            tiles, n_tiles, _, _ = meta.attn_split(1)
-            a.tiles, a.n_tiles = tiles.data_ptr(), n_tiles
-            _ok(lib().ragged_paged_attn_mfma_wide(a, meta.c(), _stream()), "paged_attn_mfma_wide")
+            # rows too wide for the row-wise kernel's lanes: long portions as tiles of 64 rows of one head, single tokens
+            # and short portions with 16 heads of a row side by side, both on the matrix cores
+            tiles, n_tiles, rows, n_rows = meta.attn_split(self.mfma_min_rows)
+            if n_tiles:
+                a.tiles, a.n_tiles = tiles.data_ptr(), n_tiles
+                _ok(lib().ragged_paged_attn_mfma_wide(a, meta.c(), _stream()), "paged_attn_mfma_wide")
+            if n_rows:
+                a.rows, a.n_rows = rows.data_ptr(), n_rows
+                _ok(lib().ragged_paged_attn_mfma_heads(a, meta.c(), _stream()), "paged_attn_mfma_heads")
             return out
         if kpages.dtype == torch.bfloat16 and self.mfma and lib().ragged_paged_attn_mfma_ok(d, vd) and a.ldv % 8 == 0:
             # long portions on the matrix cores, single tokens and short portions row by row

@@ -502,6 +502,6 @@ def test_matrix_core_attention_with_a_sink_and_with_values_inside_the_key_rows(H
             qq = q[i, hh].bfloat16().double() if i < 190 or d > 128 else q[i, hh]
             want[i, hh] = (torch.softmax((k[js, gg] @ qq) * scale, 0) @ v[js, gg]) if sink is None else \
                 O.sink_attend(qq, k[js, gg], v[js, gg], scale, sink)
-    got = _attend_through_pages("cuda", q, k, e if shared else v, [120, 70] + [1] * 10, window=window, scale=scale, sink=sink,
+    got = _attend_through_pages("cuda", q, k, e if shared else v, [120, 64, 3, 3] + [1] * 10, window=window, scale=scale, sink=sink,
                                 dtype=torch.bfloat16)
     assert float((got - want).abs().max()) < 0.03, float((got - want).abs().max())
