@@ -302,3 +302,136 @@ extern "C" int ragged_moe_combine(const void* ys, const int* place, const float*
                                             (const T*)base, (T*)y, D, top))
   return RAGGED_LAUNCH_OK();
 }
+
+// ---------------------------------------------------------------------------------------------------------------
+// Long portions: the experts' products over rows sorted by expert, one launch for all experts (bfloat16, matrix cores).
+// moe_tile_map_kernel cuts every expert's run of rows [seg[e], seg[e + 1]) into tiles of 64 rows; the product kernel's
+// workgroup (tile, block of 256 output channels) computes out^T = W_e X^T with v_mfma_f32_16x16x32_bf16, wavefront w all 64
+// rows against channels 64 w .. 64 w + 63: a lane holds one row and four neighbouring output channels of each 16 x 16
+// block, so a row's results are stored 8 bytes at a time.  Both operands are K-contiguous in memory (weights [n][k],
+// activations [row][k]), so fragments are 16-byte loads with no staging: every weight is read once per tile, the
+// activation fragments by four wavefronts (three of four from the CU's cache); 16 matrix instructions per 8 loads.
+// src_row: the activation row behind every sorted place (null: the place itself).  ACT = 1: relu(.)^2 on the way out.
+typedef __bf16 moe_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float moe_f32x4 __attribute__((ext_vector_type(4)));
+union MoeFrag {
+  moe_bf16x8 v;
+  uint4 q;
+};
+
+constexpr int MG_ROWS = 64;       // rows of a tile
+constexpr int MG_NB = 4;          // 16-channel blocks of a wavefront: a workgroup covers 256 output channels
+
+__global__ __launch_bounds__(512) void moe_tile_map_kernel(const int* __restrict__ seg, int E, int* __restrict__ tile_e,
+                                                           int* __restrict__ tile_r0, int* __restrict__ ntiles, int max_tiles) {
+  __shared__ int first[MOE_MAX_E + 1];
+  const int e = threadIdx.x;
+  const int len = e < E ? seg[e + 1] - seg[e] : 0;
+  const int cnt = (len + MG_ROWS - 1) / MG_ROWS;
+  first[e + 1 <= MOE_MAX_E ? e + 1 : MOE_MAX_E] = cnt;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    first[0] = 0;
+    for (int i = 1; i <= E; ++i) first[i] += first[i - 1];
+    *ntiles = first[E] < max_tiles ? first[E] : max_tiles;
+  }
+  __syncthreads();
+  if (e < E)
+    for (int j = 0; j < cnt; ++j)
+      if (first[e] + j < max_tiles) {
+        tile_e[first[e] + j] = e;
+        tile_r0[first[e] + j] = seg[e] + j * MG_ROWS;
+      }
+}
+
+template <int ACT>
+__global__ __launch_bounds__(256) void moe_grouped_gemm_kernel(const bf16* __restrict__ X, int64_t ldx, const int* __restrict__ src_row,
+                                                               const bf16* __restrict__ W, bf16* __restrict__ out,
+                                                               const int* __restrict__ seg, const int* __restrict__ tile_e,
+                                                               const int* __restrict__ tile_r0, const int* __restrict__ ntiles,
+                                                               int N, int K) {
+  const int tile = blockIdx.x;
+  if (tile >= *ntiles) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int lq = lane & 15, g4 = lane >> 4;
+  const int e = tile_e[tile], r0 = tile_r0[tile], rend = seg[e + 1];
+  const int n0 = (blockIdx.y * 4 + wave) * (16 * MG_NB);   // this wavefront's 16 MG_NB output channels, all 64 rows
+  if (n0 >= N) return;                                     // (no barrier in this kernel)
+  constexpr int RB = MG_ROWS / 16;
+  const bf16* xrow[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = r0 + 16 * rb + lq;
+    const int place = row < rend ? row : r0;
+    xrow[rb] = X + (int64_t)(src_row ? src_row[place] : place) * ldx;
+  }
+  const bf16* wbase = W + ((int64_t)e * N + n0) * K;
+  moe_f32x4 acc[RB][MG_NB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int nb = 0; nb < MG_NB; ++nb) acc[rb][nb] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const int k = k0 + 8 * g4;
+    MoeFrag xf[RB], wf[MG_NB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) xf[rb].q = k < K ? *reinterpret_cast<const uint4*>(xrow[rb] + k) : uint4{0, 0, 0, 0};
+#pragma unroll
+    for (int nb = 0; nb < MG_NB; ++nb) {
+      const int n = n0 + 16 * nb + lq;
+      wf[nb].q = (k < K && n < N) ? *reinterpret_cast<const uint4*>(wbase + (int64_t)(16 * nb + lq) * K + k) : uint4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int nb = 0; nb < MG_NB; ++nb)
+        acc[rb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[nb].v, xf[rb].v, acc[rb][nb], 0, 0, 0);
+  }
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = r0 + 16 * rb + lq;
+    if (row >= rend) continue;
+    bf16* orow = out + (int64_t)row * N + n0;
+#pragma unroll
+    for (int nb = 0; nb < MG_NB; ++nb) {
+      const int n = 16 * nb + 4 * g4;
+      if (n0 + n < N) {                                    // N is a multiple of 16: four channels are in or out together
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          v[i] = acc[rb][nb][i];
+          if (ACT == 1) { v[i] = fmaxf(v[i], 0.f); v[i] *= v[i]; }
+        }
+        uint2 w;
+        w.x = (uint32_t)from_f<bf16>(v[0]).b | ((uint32_t)from_f<bf16>(v[1]).b << 16);
+        w.y = (uint32_t)from_f<bf16>(v[2]).b | ((uint32_t)from_f<bf16>(v[3]).b << 16);
+        *reinterpret_cast<uint2*>(orow + n) = w;
+      }
+    }
+  }
+}
+
+// 1 when the grouped product serves these sizes (bfloat16 only)
+extern "C" int ragged_moe_grouped_ok(int N, int K, int E) { return N % 16 == 0 && K % 8 == 0 && E <= MOE_MAX_E; }
+
+extern "C" int ragged_moe_tile_map(const int* seg, int E, int* tile_e, int* tile_r0, int* ntiles, int max_tiles, hipStream_t st) {
+  if (E <= 0 || E > MOE_MAX_E || max_tiles <= 0) return -1;
+  hipLaunchKernelGGL(moe_tile_map_kernel, dim3(1), dim3(512), 0, st, seg, E, tile_e, tile_r0, ntiles, max_tiles);
+  return RAGGED_LAUNCH_OK();
+}
+
+// out[place, :N] = act(X[src_row[place], :K] . W[expert of the place][:N, :K]^T) for all sorted places
+extern "C" int ragged_moe_grouped_gemm(const void* X, int64_t ldx, const int* src_row, const void* W, void* out, const int* seg,
+                                       const int* tile_e, const int* tile_r0, const int* ntiles, int max_tiles, int N, int K, int E,
+                                       int act, hipStream_t st) {
+  if (max_tiles <= 0 || !ragged_moe_grouped_ok(N, K, E) || N <= 0 || K <= 0 || ldx < K || ldx % 8) return -1;
+  const dim3 grid(max_tiles, (N + 64 * MG_NB - 1) / (64 * MG_NB));
+  if (act == 1)
+    hipLaunchKernelGGL((moe_grouped_gemm_kernel<1>), grid, dim3(256), 0, st, (const bf16*)X, ldx, src_row, (const bf16*)W, (bf16*)out,
+                       seg, tile_e, tile_r0, ntiles, N, K);
+  else
+    hipLaunchKernelGGL((moe_grouped_gemm_kernel<0>), grid, dim3(256), 0, st, (const bf16*)X, ldx, src_row, (const bf16*)W, (bf16*)out,
+                       seg, tile_e, tile_r0, ntiles, N, K);
+  return RAGGED_LAUNCH_OK();
+}

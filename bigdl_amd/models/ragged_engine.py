@@ -292,6 +292,9 @@ class RaggedDecoder:
             base = F.linear(ops.relu2(F.linear(xa, lt.w_sup)), lt.w_sdn)
         if meta.T * f.top < self.moe_dense_rows * f.experts:
             return ops.moe_rows(xa, idx, wts, lt.w_up, lt.w_dn, base)
+        y = ops.moe_sorted(xa, idx, wts, lt.w_up, lt.w_dn, base)                # bfloat16: one grouped product per projection
+        if y is not None:
+            return y
         # rows sorted by expert: one gather, two library products per expert on its run of rows, one weighted sum per row
         T, top = meta.T, f.top
         order = idx.view(-1).sort(stable=True)

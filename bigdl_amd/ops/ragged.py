@@ -97,6 +97,9 @@ def lib():
         L.ragged_moe_route.argtypes = [vp, i64, vp, vp, vp, i64, ci, ci, ci, ci, ci, cf, ci, vp]
         L.ragged_relu2.argtypes = [vp, vp, i64, ci, vp]
         L.ragged_moe_combine.argtypes = [vp, vp, vp, vp, vp, i64, ci, ci, ci, vp]
+        L.ragged_moe_grouped_ok.argtypes = [ci, ci, ci]
+        L.ragged_moe_tile_map.argtypes = [vp, ci, vp, vp, vp, ci, vp]
+        L.ragged_moe_grouped_gemm.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
         L.ragged_moe_rows.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, i64, ci, ci, ci, ci, vp]
         L.ragged_hgrn2_chunk_decay.argtypes = [vp, vp, vp, ci, ci, vp]
         L.ragged_hgrn2_chunk_combine.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, vp]
@@ -255,7 +258,7 @@ class HipOps:
     name = "hip"
     mfma = os.environ.get("BIGDL_RAGGED_MFMA", "1") != "0"      # 0: every row through the row-wise attention kernel
     mfma_min_rows = 8
-    scan_chunk = 256          # portions of at least twice this many tokens run their recurrence in chunks
+    scan_chunk = 128          # portions of at least twice this many tokens run their recurrence in chunks
 
     def before_recording(self, meta):
         """Host-built tables a step needs (pinned allocations and copies cannot be recorded into a graph)."""
@@ -519,6 +522,40 @@ class HipOps:
                                    keep, top, scale, _DT[xa.dtype], _stream()), "moe_route")
         return idx, wts
 
+    def moe_sorted(self, xa, idx, wts, w_up, w_dn, base):
+        """The experts of long bfloat16 portions without a word to the host: (row, choice) pairs sorted by expert, every
+        expert's run cut into 64-row tiles on the device, one grouped matrix-core product for all up projections (relu^2
+        on the way out) and one for all down projections, then every row's weighted sum.  None when the sizes are not
+        served (the caller then runs the experts one by one)."""
+        T, D = xa.shape
+        E, ff, top = w_up.shape[0], w_up.shape[1], idx.shape[1]
+        L = lib()
+        if xa.dtype != torch.bfloat16 or not (L.ragged_moe_grouped_ok(ff, D, E) and L.ragged_moe_grouped_ok(D, ff, E)) \
+                or xa.stride(0) % 8 or w_up.shape != (E, ff, D) or w_dn.shape != (E, D, ff) or not w_up.is_contiguous() \
+                or not w_dn.is_contiguous() or w_up.dtype != xa.dtype or w_dn.dtype != xa.dtype:
+            return None
+        _act(xa, w_up, w_dn, base)
+        M = T * top
+        order = idx.view(-1).sort(stable=True)
+        pair = order.indices                                    # pair t * top + j at every sorted place
+        seg = torch.zeros(E + 1, dtype=torch.int32, device=xa.device)
+        seg[1:] = torch.bincount(order.values, minlength=E).cumsum(0)
+        src = (pair // top).to(torch.int32)
+        place = torch.empty(M, dtype=torch.int32, device=xa.device)
+        place[pair] = torch.arange(M, dtype=torch.int32, device=xa.device)
+        max_tiles = M // 64 + E
+        tiles = torch.empty(2 * max_tiles + 1, dtype=torch.int32, device=xa.device)
+        te, tr, nt = tiles[:max_tiles], tiles[max_tiles:2 * max_tiles], tiles[2 * max_tiles:]
+        st = _stream()
+        _ok(L.ragged_moe_tile_map(seg.data_ptr(), E, te.data_ptr(), tr.data_ptr(), nt.data_ptr(), max_tiles, st), "moe_tile_map")
+        A = torch.empty(M, ff, dtype=xa.dtype, device=xa.device)
+        ys = torch.empty(M, D, dtype=xa.dtype, device=xa.device)
+        _ok(L.ragged_moe_grouped_gemm(xa.data_ptr(), xa.stride(0), src.data_ptr(), w_up.data_ptr(), A.data_ptr(), seg.data_ptr(),
+                                      te.data_ptr(), tr.data_ptr(), nt.data_ptr(), max_tiles, ff, D, E, 1, st), "moe_grouped_gemm (up)")
+        _ok(L.ragged_moe_grouped_gemm(A.data_ptr(), ff, None, w_dn.data_ptr(), ys.data_ptr(), seg.data_ptr(), te.data_ptr(),
+                                      tr.data_ptr(), nt.data_ptr(), max_tiles, D, ff, E, 0, st), "moe_grouped_gemm (down)")
+        return self.moe_combine(ys, place.view(T, top), wts, base)
+
     def moe_combine(self, ys, place, wts, base):
         """y[t] = base[t] + sum_j wts[t, j] * ys[place[t, j]]"""
         _act(ys, base)
@@ -736,6 +773,9 @@ class TorchOps:
         kept.scatter_(1, best.topk(keep, -1).indices, True)
         idx = s.masked_fill(~kept.repeat_interleave(E // groups, 1), -1.0).topk(top, -1).indices
         return idx.to(torch.int32), s.gather(1, idx) * scale
+
+    def moe_sorted(self, xa, idx, wts, w_up, w_dn, base):
+        return None                                             # (the host statements run the experts one by one)
 
     def moe_combine(self, ys, place, wts, base):
         y = torch.zeros(place.shape[0], ys.shape[1]) if base is None else base.float().clone()

@@ -505,3 +505,34 @@ def test_matrix_core_attention_with_a_sink_and_with_values_inside_the_key_rows(H
     got = _attend_through_pages("cuda", q, k, e if shared else v, [120, 64, 3, 3] + [1] * 10, window=window, scale=scale, sink=sink,
                                 dtype=torch.bfloat16)
     assert float((got - want).abs().max()) < 0.03, float((got - want).abs().max())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,D,ff,experts,top,count,keep", [(300, 64, 48, 10, 3, 5, 2), (1000, 256, 112, 64, 6, 8, 4), (70, 80, 16, 3, 3, 1, 1),
+                                                         (129, 128, 128, 40, 1, 1, 1)])
+def test_grouped_expert_product_on_sorted_rows(T, D, ff, experts, top, count, keep):
+    """bfloat16 long portions: every expert's run of sorted rows through the grouped matrix-core product, against float64
+    on the same bfloat16 inputs and against the row-wise kernels"""
+    g = torch.Generator().manual_seed(91)
+    ops = R.ops_for("cuda")
+    x = (torch.randn(T + 3, D + 8, generator=g)).bfloat16().cuda()[3:, :D]                    # rows with a stride of their own
+    x = x if x.stride(0) % 8 == 0 else x.contiguous()
+    wr = (torch.randn(experts, D, generator=g) * 0.4).cuda()
+    up = (torch.randn(experts, ff, D, generator=g) * 0.2).bfloat16().cuda()
+    dn = (torch.randn(experts, D, ff, generator=g) * 0.2).bfloat16().cuda()
+    base = torch.randn(T, D, generator=g).bfloat16().cuda()
+    idx, wts = ops.moe_route(x, wr, count, keep, top, 1.3)
+    got = ops.moe_sorted(x, idx, wts, up, dn, base)
+    assert got is not None
+    assert ops.moe_sorted(x[:, :D - 4].contiguous(), idx, wts, up[:, :, :D - 4].contiguous(), dn[:, :D - 4].contiguous(), None) is None
+    rows = ops.moe_rows(x, idx, wts, up, dn, base)
+    ref = base.double().cpu()
+    xd, upd, dnd = x.double().cpu(), up.double().cpu(), dn.double().cpu()
+    for t in range(T):
+        for j in range(top):
+            e = int(idx[t, j])
+            a = torch.relu(upd[e] @ xd[t]).pow(2).bfloat16().double()
+            ref[t] += float(wts[t, j]) * (dnd[e] @ a).bfloat16().double()
+    scale = float(ref.abs().max())
+    assert float((got.double().cpu() - ref).abs().max()) < 0.02 * scale
+    assert float((rows.double().cpu() - ref).abs().max()) < 0.02 * scale
