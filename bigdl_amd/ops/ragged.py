@@ -365,7 +365,7 @@ class HipOps:
                                     out.data_ptr(), H, d, vd, oc, meta.c(), dt, st), "hgrn2_scan")
             return out
         # long portions: chunks scanned side by side from zero, chunk-start states chained, chunks scanned again from them
-        nc, cstart, zeros, ones, cid, cfirst, last = meta.chunks(self.scan_chunk)
+        nc, cstart, zeros, ones, cid, cfirst, last = meta.chunks(self._chunk_length(meta, H, d, vd))
         local = torch.empty(nc, H, d, vd, dtype=torch.float32, device=P.device)
         begin = torch.empty_like(local)
         decay = torch.empty(nc, H * d, dtype=torch.float32, device=P.device)
@@ -383,6 +383,23 @@ class HipOps:
         slots = torch.tensor([s[0] for s in meta.seqs], dtype=torch.int64, device=P.device)
         state[slots] = begin[torch.tensor(last, dtype=torch.int64, device=P.device)]     # every sequence's end state
         return out
+
+    scan_resident = 512       # workgroups of the scan that run at one time (two per CU)
+
+    def _chunk_length(self, meta, H, d, vd):
+        """Tokens per chunk of a long scan: a pass takes (rounds of resident workgroups) x (tokens of a chunk), so the
+        length is chosen for the fewest token steps in a row; among equals the longest (fewer chunk states to chain)."""
+        R = 1
+        while R * 32 < d:
+            R *= 2
+        blocks = -(-vd // (4 * (64 // R)))                   # column blocks of a head
+        best = None
+        for length in (256, 224, 192, 160, 128, 96, 64):
+            chunks = sum(-(-n // length) for _, _, n, _ in meta.seqs)
+            cost = -(-(chunks * H * blocks) // self.scan_resident) * min(length, max(n for _, _, n, _ in meta.seqs))
+            if best is None or cost < best[0]:
+                best = (cost, length)
+        return best[1]
 
     def row_norm(self, x, w, eps, act):
         _f32(x, w)
