@@ -308,9 +308,10 @@ extern "C" int ragged_moe_combine(const void* ys, const int* place, const float*
 // moe_tile_map_kernel cuts every expert's run of rows [seg[e], seg[e + 1]) into tiles of 64 rows; the product kernel's
 // workgroup (tile, block of 256 output channels) computes out^T = W_e X^T with v_mfma_f32_16x16x32_bf16, wavefront w all 64
 // rows against channels 64 w .. 64 w + 63: a lane holds one row and four neighbouring output channels of each 16 x 16
-// block, so a row's results are stored 8 bytes at a time.  Both operands are K-contiguous in memory (weights [n][k],
-// activations [row][k]), so fragments are 16-byte loads with no staging: every weight is read once per tile, the
-// activation fragments by four wavefronts (three of four from the CU's cache); 16 matrix instructions per 8 loads.
+// block, so a row's results are stored 8 bytes at a time.  K runs in steps of 64 channels: the step's weight tile
+// [256][64] and activation tile [64][64] are read by the whole workgroup in 128-byte row pieces into registers while the
+// previous step's matrix instructions run, stored to the other of two LDS buffers, and read back as fragments (both
+// operands are K-contiguous, so a fragment is one 16-byte LDS read); one barrier per step.
 // src_row: the activation row behind every sorted place (null: the place itself).  ACT = 1: relu(.)^2 on the way out.
 typedef __bf16 moe_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float moe_f32x4 __attribute__((ext_vector_type(4)));
@@ -344,50 +345,87 @@ __global__ __launch_bounds__(512) void moe_tile_map_kernel(const int* __restrict
       }
 }
 
+constexpr int MG_K = 64;          // channels of a K step
+constexpr int MG_LD = MG_K + 8;   // LDS row stride in elements: rows stay 16-byte aligned and neighbouring rows shift banks
+constexpr int MG_N = 64 * MG_NB;  // output channels of a workgroup
+
 template <int ACT>
 __global__ __launch_bounds__(256) void moe_grouped_gemm_kernel(const bf16* __restrict__ X, int64_t ldx, const int* __restrict__ src_row,
                                                                const bf16* __restrict__ W, bf16* __restrict__ out,
                                                                const int* __restrict__ seg, const int* __restrict__ tile_e,
                                                                const int* __restrict__ tile_r0, const int* __restrict__ ntiles,
                                                                int N, int K) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t tiles[];   // 2 x { W [MG_N][MG_LD], X [MG_ROWS][MG_LD] }
   const int tile = blockIdx.x;
-  if (tile >= *ntiles) return;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (tile >= *ntiles) return;                             // (the whole workgroup leaves: no barrier is left waiting)
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int lq = lane & 15, g4 = lane >> 4;
   const int e = tile_e[tile], r0 = tile_r0[tile], rend = seg[e + 1];
-  const int n0 = (blockIdx.y * 4 + wave) * (16 * MG_NB);   // this wavefront's 16 MG_NB output channels, all 64 rows
-  if (n0 >= N) return;                                     // (no barrier in this kernel)
-  constexpr int RB = MG_ROWS / 16;
-  const bf16* xrow[RB];
+  const int nw = blockIdx.y * MG_N;                        // the workgroup's first output channel
+  constexpr int RB = MG_ROWS / 16, BUF = (MG_N + MG_ROWS) * MG_LD;
+  constexpr int WP = MG_N * (MG_K / 8) / 256, XP = MG_ROWS * (MG_K / 8) / 256;   // 16-byte pieces per thread
+  // loaders: piece p of a tile = (row p / 8, channels 8 (p % 8) ..): eight neighbouring threads read 128 bytes of a row
+  const bf16* wsrc[WP];
+  const bf16* xsrc[XP];
 #pragma unroll
-  for (int rb = 0; rb < RB; ++rb) {
-    const int row = r0 + 16 * rb + lq;
-    const int place = row < rend ? row : r0;
-    xrow[rb] = X + (int64_t)(src_row ? src_row[place] : place) * ldx;
+  for (int u = 0; u < WP; ++u) {
+    const int n = nw + ((tid + 256 * u) >> 3);
+    wsrc[u] = n < N ? W + ((int64_t)e * N + n) * K : nullptr;
   }
-  const bf16* wbase = W + ((int64_t)e * N + n0) * K;
+#pragma unroll
+  for (int u = 0; u < XP; ++u) {
+    const int row = r0 + ((tid + 256 * u) >> 3);
+    const int place = row < rend ? row : r0;
+    xsrc[u] = X + (int64_t)(src_row ? src_row[place] : place) * ldx;
+  }
+  const int pc = 8 * (tid & 7);
+  uint4 wreg[WP], xreg[XP];
+  auto gload = [&](int k0) {
+    const int k = k0 + pc;
+#pragma unroll
+    for (int u = 0; u < WP; ++u)
+      wreg[u] = (wsrc[u] && k < K) ? *reinterpret_cast<const uint4*>(wsrc[u] + k) : uint4{0, 0, 0, 0};
+#pragma unroll
+    for (int u = 0; u < XP; ++u) xreg[u] = k < K ? *reinterpret_cast<const uint4*>(xsrc[u] + k) : uint4{0, 0, 0, 0};
+  };
+  auto lstore = [&](uint16_t* buf) {
+#pragma unroll
+    for (int u = 0; u < WP; ++u) *reinterpret_cast<uint4*>(buf + ((tid + 256 * u) >> 3) * MG_LD + pc) = wreg[u];
+#pragma unroll
+    for (int u = 0; u < XP; ++u) *reinterpret_cast<uint4*>(buf + (MG_N + ((tid + 256 * u) >> 3)) * MG_LD + pc) = xreg[u];
+  };
   moe_f32x4 acc[RB][MG_NB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
     for (int nb = 0; nb < MG_NB; ++nb) acc[rb][nb] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 2
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    const int k = k0 + 8 * g4;
-    MoeFrag xf[RB], wf[MG_NB];
+  gload(0);
+  lstore(tiles);
+  __syncthreads();
+  int cur = 0;
+  for (int k0 = 0; k0 < K; k0 += MG_K) {
+    const bool more = k0 + MG_K < K;
+    if (more) gload(k0 + MG_K);                            // in flight during this step's matrix instructions
+    const uint16_t* wt = tiles + cur * BUF + (64 * wave) * MG_LD;
+    const uint16_t* xt = tiles + cur * BUF + MG_N * MG_LD;
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) xf[rb].q = k < K ? *reinterpret_cast<const uint4*>(xrow[rb] + k) : uint4{0, 0, 0, 0};
+    for (int ks = 0; ks < MG_K / 32; ++ks) {
+      MoeFrag xf[RB], wf[MG_NB];
 #pragma unroll
-    for (int nb = 0; nb < MG_NB; ++nb) {
-      const int n = n0 + 16 * nb + lq;
-      wf[nb].q = (k < K && n < N) ? *reinterpret_cast<const uint4*>(wbase + (int64_t)(16 * nb + lq) * K + k) : uint4{0, 0, 0, 0};
+      for (int rb = 0; rb < RB; ++rb) xf[rb].q = *reinterpret_cast<const uint4*>(xt + (16 * rb + lq) * MG_LD + 32 * ks + 8 * g4);
+#pragma unroll
+      for (int nb = 0; nb < MG_NB; ++nb) wf[nb].q = *reinterpret_cast<const uint4*>(wt + (16 * nb + lq) * MG_LD + 32 * ks + 8 * g4);
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int nb = 0; nb < MG_NB; ++nb)
+          acc[rb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[nb].v, xf[rb].v, acc[rb][nb], 0, 0, 0);
     }
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-      for (int nb = 0; nb < MG_NB; ++nb)
-        acc[rb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[nb].v, xf[rb].v, acc[rb][nb], 0, 0, 0);
+    if (more) lstore(tiles + (cur ^ 1) * BUF);             // (its last readers passed the barrier of the step before)
+    __syncthreads();
+    cur ^= 1;
   }
+  const int n0 = nw + 64 * wave;
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int row = r0 + 16 * rb + lq;
@@ -426,12 +464,20 @@ extern "C" int ragged_moe_grouped_gemm(const void* X, int64_t ldx, const int* sr
                                        const int* tile_e, const int* tile_r0, const int* ntiles, int max_tiles, int N, int K, int E,
                                        int act, hipStream_t st) {
   if (max_tiles <= 0 || !ragged_moe_grouped_ok(N, K, E) || N <= 0 || K <= 0 || ldx < K || ldx % 8) return -1;
-  const dim3 grid(max_tiles, (N + 64 * MG_NB - 1) / (64 * MG_NB));
+  const dim3 grid(max_tiles, (N + MG_N - 1) / MG_N);
+  const size_t lds = 2 * (size_t)(MG_N + MG_ROWS) * MG_LD * sizeof(uint16_t);
+  static bool raised = false;                               // two tiles above 64 KB: the limit is raised once per kernel
+  if (!raised) {
+    if (hipFuncSetAttribute((const void*)moe_grouped_gemm_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess ||
+        hipFuncSetAttribute((const void*)moe_grouped_gemm_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return -3;
+    raised = true;
+  }
   if (act == 1)
-    hipLaunchKernelGGL((moe_grouped_gemm_kernel<1>), grid, dim3(256), 0, st, (const bf16*)X, ldx, src_row, (const bf16*)W, (bf16*)out,
+    hipLaunchKernelGGL((moe_grouped_gemm_kernel<1>), grid, dim3(256), lds, st, (const bf16*)X, ldx, src_row, (const bf16*)W, (bf16*)out,
                        seg, tile_e, tile_r0, ntiles, N, K);
   else
-    hipLaunchKernelGGL((moe_grouped_gemm_kernel<0>), grid, dim3(256), 0, st, (const bf16*)X, ldx, src_row, (const bf16*)W, (bf16*)out,
+    hipLaunchKernelGGL((moe_grouped_gemm_kernel<0>), grid, dim3(256), lds, st, (const bf16*)X, ldx, src_row, (const bf16*)W, (bf16*)out,
                        seg, tile_e, tile_r0, ntiles, N, K);
   return RAGGED_LAUNCH_OK();
 }
