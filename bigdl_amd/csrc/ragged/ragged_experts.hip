@@ -345,7 +345,7 @@ __global__ __launch_bounds__(512) void moe_tile_map_kernel(const int* __restrict
       }
 }
 
-constexpr int MG_K = 64;          // channels of a K step
+constexpr int MG_K = 32;          // channels of a K step
 constexpr int MG_LD = MG_K + 8;   // LDS row stride in elements: rows stay 16-byte aligned and neighbouring rows shift banks
 constexpr int MG_N = 64 * MG_NB;  // output channels of a workgroup
 
@@ -363,22 +363,23 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_kernel(const bf16* __res
   const int e = tile_e[tile], r0 = tile_r0[tile], rend = seg[e + 1];
   const int nw = blockIdx.y * MG_N;                        // the workgroup's first output channel
   constexpr int RB = MG_ROWS / 16, BUF = (MG_N + MG_ROWS) * MG_LD;
-  constexpr int WP = MG_N * (MG_K / 8) / 256, XP = MG_ROWS * (MG_K / 8) / 256;   // 16-byte pieces per thread
+  constexpr int PPR = MG_K / 8;                            // 16-byte pieces of a tile row
+  constexpr int WP = MG_N * PPR / 256, XP = MG_ROWS * PPR / 256;   // pieces per thread
   // loaders: piece p of a tile = (row p / 8, channels 8 (p % 8) ..): eight neighbouring threads read 128 bytes of a row
   const bf16* wsrc[WP];
   const bf16* xsrc[XP];
 #pragma unroll
   for (int u = 0; u < WP; ++u) {
-    const int n = nw + ((tid + 256 * u) >> 3);
+    const int n = nw + (tid + 256 * u) / PPR;
     wsrc[u] = n < N ? W + ((int64_t)e * N + n) * K : nullptr;
   }
 #pragma unroll
   for (int u = 0; u < XP; ++u) {
-    const int row = r0 + ((tid + 256 * u) >> 3);
+    const int row = r0 + (tid + 256 * u) / PPR;
     const int place = row < rend ? row : r0;
     xsrc[u] = X + (int64_t)(src_row ? src_row[place] : place) * ldx;
   }
-  const int pc = 8 * (tid & 7);
+  const int pc = 8 * (tid % PPR);
   uint4 wreg[WP], xreg[XP];
   auto gload = [&](int k0) {
     const int k = k0 + pc;
@@ -390,9 +391,9 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_kernel(const bf16* __res
   };
   auto lstore = [&](uint16_t* buf) {
 #pragma unroll
-    for (int u = 0; u < WP; ++u) *reinterpret_cast<uint4*>(buf + ((tid + 256 * u) >> 3) * MG_LD + pc) = wreg[u];
+    for (int u = 0; u < WP; ++u) *reinterpret_cast<uint4*>(buf + ((tid + 256 * u) / PPR) * MG_LD + pc) = wreg[u];
 #pragma unroll
-    for (int u = 0; u < XP; ++u) *reinterpret_cast<uint4*>(buf + (MG_N + ((tid + 256 * u) >> 3)) * MG_LD + pc) = xreg[u];
+    for (int u = 0; u < XP; ++u) *reinterpret_cast<uint4*>(buf + (MG_N + (tid + 256 * u) / PPR) * MG_LD + pc) = xreg[u];
   };
   moe_f32x4 acc[RB][MG_NB];
 #pragma unroll
