@@ -103,8 +103,9 @@ class YuanAttention(nn.Module):
         self.k_proj = nn.Linear(c, c, bias=False)
         self.v_proj = nn.Linear(c, c, bias=False)
         self.o_proj = nn.Linear(c, c, bias=False)
-        inv = 1.0 / (config.rope_theta ** (torch.arange(0, self.head_dim, 2).float() / self.head_dim))
-        self.register_buffer("inv_freq", inv, persistent=False)
+        # (not a buffer: a checkpoint loader that builds the module on the meta device hands non-persistent buffers back
+        # as uninitialised memory)
+        self.rope_theta = float(config.rope_theta)
 
     def forward(self, x, position_ids, past=None, attention_mask=None):
         b, t, c = x.shape
@@ -116,7 +117,8 @@ class YuanAttention(nn.Module):
         f = self.lf_gate(x, before)
         qk = torch.cat([self.q_proj(f), self.k_proj(f)], -1).view(b, t, h, 2 * d)
         q, k = (s.transpose(1, 2) for s in torch.chunk(qk, 2, -1))
-        ang = position_ids[:, :, None].float() * self.inv_freq[None, None, :].float()        # [B, T, d/2]
+        inv_freq = 1.0 / (self.rope_theta ** (torch.arange(0, d, 2, device=x.device).float() / d))
+        ang = position_ids[:, :, None].float() * inv_freq[None, None, :]                      # [B, T, d/2]
         cos, sin = (torch.cat([fn(ang), fn(ang)], -1)[:, None].to(q.dtype) for fn in (torch.cos, torch.sin))
         q, k = q * cos + _rotate_half(q) * sin, k * cos + _rotate_half(k) * sin
         if past is not None:
